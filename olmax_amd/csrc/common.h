@@ -1,0 +1,96 @@
+// Shared device/host helpers for the gfx950 kernels of libolmax_hip.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+typedef __bf16 bf16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define OLMAX_OK 0
+#define OLMAX_ERR_ARG (-1)
+#define OLMAX_ERR_SHAPE (-2)
+#define OLMAX_ERR_ALIGN (-3)
+#define OLMAX_ERR_LAUNCH (-4)
+#define OLMAX_ERR_WORKSPACE (-5)
+
+// Thread-local last error message (returned by olmax_last_error_string()).
+int olmax_set_error(int code, const char* fmt, ...);
+
+#define OLMAX_CHECK(cond, code, ...)                    \
+  do {                                                  \
+    if (!(cond)) return olmax_set_error(code, __VA_ARGS__); \
+  } while (0)
+
+#define OLMAX_LAUNCH_CHECK()                                                    \
+  do {                                                                          \
+    hipError_t e__ = hipGetLastError();                                         \
+    if (e__ != hipSuccess)                                                      \
+      return olmax_set_error(OLMAX_ERR_LAUNCH, "%s:%d launch failed: %s", __FILE__, __LINE__, \
+                             hipGetErrorString(e__));                           \
+  } while (0)
+
+static inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+__device__ __forceinline__ float bf2f(bf16 x) { return (float)x; }
+__device__ __forceinline__ bf16 f2bf(float x) { return (bf16)x; }
+
+// 128-bit vector of 8 bf16, as raw words for loads/stores.
+union Pack8 {
+  u32x4 u;
+  bf16x8 v;
+  bf16 e[8];
+};
+union Pack4 {
+  u32x2 u;
+  bf16x4 v;
+  bf16 e[4];
+};
+
+// Wave64 all-reduce (sum) by xor shuffles.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Block-wide sum for blocks of NW waves; `red` is NW floats of LDS. All threads get the result.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  if (NW == 1) return v;
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < NW; i++) t += red[i];
+  return t;
+}
+template <int NW>
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  if (NW == 1) return v;
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float t = red[0];
+#pragma unroll
+  for (int i = 1; i < NW; i++) t = fmaxf(t, red[i]);
+  return t;
+}

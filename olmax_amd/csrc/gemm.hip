@@ -1,0 +1,346 @@
+// bf16 MFMA GEMM for gfx950 (MI355X): C[M,N] = A[M,K] * B[N,K]^T (+ R), fp32 accumulate.
+//
+// Replaces the cuBLASLt calls XLA issues for olmax.nn.functional.linear
+// (reference src/olmax/nn/functional.py:14-27) and for the two transposed
+// products its autodiff derives (dX = dY W, dW = dY^T X).
+//
+// One kernel template covers the three operand storage combinations:
+//   A "KC": A[m*lda + k]   (reduction dim contiguous)   A "MC": A[k*lda + m]
+//   B "KC": B[n*ldb + k]                                 B "NC": B[k*ldb + n]
+// forward  Y = X W^T      : A=X  (KC), B=W  (KC)
+// dX = dY W               : A=dY (KC), B=W  (NC)   (reduction over out-features)
+// dW = dY^T X             : A=dY (MC), B=X  (NC)   (reduction over tokens)
+//
+// Tiling: BM x BN x 64 block tile, 64-lane waves each owning a WM x WN sub-tile as
+// (WM/32) x (WN/32) v_mfma_f32_32x32x16_bf16 accumulators. Operand tiles are staged
+// through LDS with a register-held prefetch of the next k-tile (double buffered LDS,
+// one barrier per k-tile). K-contiguous tiles live in LDS as [rows][64] with the 16-byte
+// chunk index XOR-swizzled by row so ds_read_b128 is bank-conflict free; M/N-contiguous
+// tiles live as [64][rows] and are read with ds_read_b64_tr_b16, the gfx950 transposing
+// LDS load, which hands each lane 4 consecutive reduction-dim elements of its column.
+//
+// Workgroup -> tile mapping is XCD aware: hardware deals consecutive workgroup ids
+// round-robin over the 8 XCDs, so id i is remapped to (i % 8) * (grid/8) + i / 8, giving
+// every XCD one contiguous run of tiles; runs walk the tile grid in column groups so that
+// the A row-panels and B column-panels a single L2 sees are re-used.
+#include "common.h"
+
+namespace {
+
+constexpr int BK = 64;
+
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
+    const bf16* __restrict__ A, const bf16* __restrict__ B, void* __restrict__ Cv,
+    const bf16* __restrict__ R, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+    int64_t ldr, int tiles_m, int tiles_n) {
+  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int WAVES_N = BN / WN;
+  constexpr int A_CHUNKS = BM * BK / 8 / NT;  // 16-byte chunks per thread per k-tile
+  constexpr int B_CHUNKS = BN * BK / 8 / NT;
+  static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "tile too small for thread count");
+  constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // layout: [stage][A tile | B tile]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  // ---- XCD-aware tile assignment ----
+  const int nwg = gridDim.x;
+  int pid = blockIdx.x;
+  {
+    const int per = nwg >> 3;
+    if ((nwg & 7) == 0) pid = (pid & 7) * per + (pid >> 3);
+  }
+  // column-grouped walk: groups of GM row-tiles, sweep N inside a group
+  constexpr int GM = 8;
+  const int group_sz = GM * tiles_n;
+  const int gid = pid / group_sz;
+  const int first_m = gid * GM;
+  const int gm = min(tiles_m - first_m, GM);
+  const int tile_m = first_m + (pid % group_sz) % gm;
+  const int tile_n = (pid % group_sz) / gm;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  // ---- per-thread global source addresses ----
+  const bf16* a_src[A_CHUNKS];
+  int a_dst[A_CHUNKS];
+#pragma unroll
+  for (int i = 0; i < A_CHUNKS; i++) {
+    const int q = i * NT + tid;
+    if (A_KC) {
+      const int row = q >> 3, kc = q & 7;
+      a_src[i] = A + (int64_t)(m0 + row) * lda + kc * 8;
+      a_dst[i] = row * 128 + ((kc ^ (row & 7)) << 4);
+    } else {
+      constexpr int CPR = BM / 8;  // chunks per k-row
+      const int kr = q / CPR, mc = q % CPR;
+      a_src[i] = A + (int64_t)kr * lda + m0 + mc * 8;
+      a_dst[i] = kr * (BM * 2) + ((mc ^ ((kr & 3) << 1)) << 4);
+    }
+  }
+  const bf16* b_src[B_CHUNKS];
+  int b_dst[B_CHUNKS];
+#pragma unroll
+  for (int i = 0; i < B_CHUNKS; i++) {
+    const int q = i * NT + tid;
+    if (B_KC) {
+      const int row = q >> 3, kc = q & 7;
+      b_src[i] = B + (int64_t)(n0 + row) * ldb + kc * 8;
+      b_dst[i] = row * 128 + ((kc ^ (row & 7)) << 4);
+    } else {
+      constexpr int CPR = BN / 8;
+      const int kr = q / CPR, nc = q % CPR;
+      b_src[i] = B + (int64_t)kr * ldb + n0 + nc * 8;
+      b_dst[i] = kr * (BN * 2) + ((nc ^ ((kr & 3) << 1)) << 4);
+    }
+  }
+  const int64_t a_step = A_KC ? (int64_t)BK : (int64_t)BK * lda;
+  const int64_t b_step = B_KC ? (int64_t)BK : (int64_t)BK * ldb;
+
+  u32x4 a_reg[A_CHUNKS], b_reg[B_CHUNKS];
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  const int KT = K / BK;
+
+  auto gload = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; i++)
+      a_reg[i] = *reinterpret_cast<const u32x4*>(a_src[i] + (int64_t)kt * a_step);
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; i++)
+      b_reg[i] = *reinterpret_cast<const u32x4*>(b_src[i] + (int64_t)kt * b_step);
+  };
+  auto lstore = [&](int stage) {
+    unsigned char* sa = smem + stage * (A_BYTES + B_BYTES);
+    unsigned char* sb = sa + A_BYTES;
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; i++) *reinterpret_cast<u32x4*>(sa + a_dst[i]) = a_reg[i];
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; i++) *reinterpret_cast<u32x4*>(sb + b_dst[i]) = b_reg[i];
+  };
+
+  // lane-constant parts of the LDS fragment addresses
+  const int l32 = lane & 31, lhi = lane >> 5;
+  // transposed-read geometry: 16-lane group g: column half = g & 1, k-group = g >> 1
+  const int j16 = lane & 15, g16 = lane >> 4;
+  const int tr_krow = ((g16 >> 1) << 3) + (j16 >> 2);        // + kk*16 (+4 for second read)
+  const int tr_col = ((g16 & 1) << 4) + ((j16 & 3) << 2);     // element offset inside 32-wide tile
+
+  auto compute = [&](int stage) {
+    const unsigned char* sa = smem + stage * (A_BYTES + B_BYTES);
+    const unsigned char* sb = sa + A_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; kk++) {
+      bf16x8 af[TM], bfr[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        if (A_KC) {
+          const int row = wm * WM + i * 32 + l32;
+          const int ch = kk * 2 + lhi;
+          af[i] = *reinterpret_cast<const bf16x8*>(sa + row * 128 + ((ch ^ (row & 7)) << 4));
+        } else {
+          const int col = wm * WM + i * 32 + tr_col;
+          Pack8 p;
+#pragma unroll
+          for (int h = 0; h < 2; h++) {
+            const int kr = kk * 16 + tr_krow + h * 4;
+            const int off = kr * (BM * 2) + (((col >> 3) ^ ((kr & 3) << 1)) << 4) + ((col & 7) << 1);
+            s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (s16x4 __attribute__((address_space(3)))*)(sa + off));
+            p.u[h * 2 + 0] = ((u32x2&)t)[0];
+            p.u[h * 2 + 1] = ((u32x2&)t)[1];
+          }
+          af[i] = p.v;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        if (B_KC) {
+          const int row = wn * WN + j * 32 + l32;
+          const int ch = kk * 2 + lhi;
+          bfr[j] = *reinterpret_cast<const bf16x8*>(sb + row * 128 + ((ch ^ (row & 7)) << 4));
+        } else {
+          const int col = wn * WN + j * 32 + tr_col;
+          Pack8 p;
+#pragma unroll
+          for (int h = 0; h < 2; h++) {
+            const int kr = kk * 16 + tr_krow + h * 4;
+            const int off = kr * (BN * 2) + (((col >> 3) ^ ((kr & 3) << 1)) << 4) + ((col & 7) << 1);
+            s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (s16x4 __attribute__((address_space(3)))*)(sb + off));
+            p.u[h * 2 + 0] = ((u32x2&)t)[0];
+            p.u[h * 2 + 1] = ((u32x2&)t)[1];
+          }
+          bfr[j] = p.v;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  for (int kt = 0; kt < KT; kt++) {
+    const int cur = kt & 1;
+    if (kt + 1 < KT) gload(kt + 1);
+    compute(cur);
+    if (kt + 1 < KT) lstore(cur ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: accumulator (lane -> column l32, rows 8*(r/4) + 4*lhi + r%4) ----
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int col = n0 + wn * WN + j * 32 + l32;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int row = m0 + wm * WM + i * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
+        float v = acc[i][j][r];
+        if (HAS_RES) v += bf2f(R[(int64_t)row * ldr + col]);
+        if (OUT_F32)
+          reinterpret_cast<float*>(Cv)[(int64_t)row * ldc + col] = v;
+        else
+          reinterpret_cast<bf16*>(Cv)[(int64_t)row * ldc + col] = f2bf(v);
+      }
+    }
+}
+
+// Bounds-checked scalar-FMA kernel for shapes the MFMA tiles do not divide
+// (the reference's own unit tests use d_model=16, seq=12). One 16x16 output tile per block.
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(
+    const bf16* __restrict__ A, const bf16* __restrict__ B, void* __restrict__ Cv,
+    const bf16* __restrict__ R, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+    int64_t ldr, int a_kc, int b_kc) {
+  __shared__ float As[16][17], Bs[16][17];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int row = blockIdx.y * 16 + ty, col = blockIdx.x * 16 + tx;
+  float acc = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    {
+      const int m = blockIdx.y * 16 + ty, k = k0 + tx;
+      As[ty][tx] = (m < M && k < K) ? bf2f(a_kc ? A[(int64_t)m * lda + k] : A[(int64_t)k * lda + m]) : 0.f;
+      const int n = blockIdx.x * 16 + ty;
+      Bs[ty][tx] = (n < N && k < K) ? bf2f(b_kc ? B[(int64_t)n * ldb + k] : B[(int64_t)k * ldb + n]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; k++) acc += As[ty][k] * Bs[tx][k];
+    __syncthreads();
+  }
+  if (row < M && col < N) {
+    if (R) acc += bf2f(R[(int64_t)row * ldr + col]);
+    if (OUT_F32)
+      reinterpret_cast<float*>(Cv)[(int64_t)row * ldc + col] = acc;
+    else
+      reinterpret_cast<bf16*>(Cv)[(int64_t)row * ldc + col] = f2bf(acc);
+  }
+}
+
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32>
+int launch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16* R, int M, int N,
+                int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldr) {
+  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  constexpr int SMEM = 2 * (BM + BN) * BK * 2;
+  auto kern = gemm_bf16_kernel<BM, BN, WM, WN, A_KC, B_KC, HAS_RES, OUT_F32>;
+  static bool attr_set = false;  // one-time, idempotent
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+    attr_set = true;
+  }
+  const int tm = M / BM, tn = N / BN;
+  hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(NT), SMEM, s, A, B, C, R, M, N, K, lda, ldb, ldc,
+                     ldr, tm, tn);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+template <bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32>
+int dispatch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16* R, int M, int N,
+                  int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldr, int tile) {
+  if (tile == 256)
+    return launch_tile<256, 256, 128, 64, A_KC, B_KC, HAS_RES, OUT_F32>(s, A, B, C, R, M, N, K, lda,
+                                                                        ldb, ldc, ldr);
+  if (tile == 257)
+    return launch_tile<256, 256, 128, 128, A_KC, B_KC, HAS_RES, OUT_F32>(s, A, B, C, R, M, N, K,
+                                                                         lda, ldb, ldc, ldr);
+  return launch_tile<128, 128, 64, 64, A_KC, B_KC, HAS_RES, OUT_F32>(s, A, B, C, R, M, N, K, lda,
+                                                                     ldb, ldc, ldr);
+}
+
+int g_force_tile = 0;
+
+}  // namespace
+
+extern "C" void olmax_gemm_set_tile(int tile) { g_force_tile = tile; }
+
+extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void* B, void* C,
+                                   const void* R, int32_t M, int32_t N, int32_t K, int64_t lda,
+                                   int64_t ldb, int64_t ldc, int64_t ldr, int32_t a_layout,
+                                   int32_t b_layout, int32_t out_f32) {
+  OLMAX_CHECK(A && B && C, OLMAX_ERR_ARG, "olmax_gemm_bf16: null operand");
+  OLMAX_CHECK(M > 0 && N > 0 && K > 0, OLMAX_ERR_SHAPE, "olmax_gemm_bf16: M,N,K must be positive (got %d,%d,%d)", M, N, K);
+  OLMAX_CHECK((a_layout == 0 || a_layout == 1) && (b_layout == 0 || b_layout == 1), OLMAX_ERR_ARG,
+              "olmax_gemm_bf16: layout flags must be 0 (reduction-contiguous) or 1");
+  const bool a_kc = a_layout == 0, b_kc = b_layout == 0;
+  OLMAX_CHECK(lda >= (a_kc ? K : M) && ldb >= (b_kc ? K : N) && ldc >= N && (!R || ldr >= N),
+              OLMAX_ERR_SHAPE, "olmax_gemm_bf16: leading dimension smaller than row length");
+  const bf16* a = (const bf16*)A;
+  const bf16* b = (const bf16*)B;
+  const bf16* r = (const bf16*)R;
+  const bool vec_ok = aligned16(A) && aligned16(B) && (lda % 8 == 0) && (ldb % 8 == 0);
+  int tile = 0;
+  if (vec_ok && K % BK == 0) {
+    if (M % 256 == 0 && N % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 128) tile = 256;
+    else if (M % 128 == 0 && N % 128 == 0) tile = 128;
+  }
+  if (g_force_tile && tile) {
+    if (g_force_tile >= 256 && M % 256 == 0 && N % 256 == 0) tile = g_force_tile;
+    if (g_force_tile == 128) tile = 128;
+  }
+  if (tile == 0) {
+    dim3 grid((N + 15) / 16, (M + 15) / 16);
+    if (out_f32)
+      hipLaunchKernelGGL(gemm_generic_kernel<true>, grid, dim3(256), 0, stream, a, b, C, r, M, N, K,
+                         lda, ldb, ldc, ldr, (int)a_kc, (int)b_kc);
+    else
+      hipLaunchKernelGGL(gemm_generic_kernel<false>, grid, dim3(256), 0, stream, a, b, C, r, M, N,
+                         K, lda, ldb, ldc, ldr, (int)a_kc, (int)b_kc);
+    OLMAX_LAUNCH_CHECK();
+    return OLMAX_OK;
+  }
+#define GO(AK, BKC)                                                                              \
+  do {                                                                                           \
+    if (r) {                                                                                     \
+      if (out_f32) return dispatch_tile<AK, BKC, true, true>(stream, a, b, C, r, M, N, K, lda, ldb, ldc, ldr, tile); \
+      return dispatch_tile<AK, BKC, true, false>(stream, a, b, C, r, M, N, K, lda, ldb, ldc, ldr, tile);             \
+    } else {                                                                                     \
+      if (out_f32) return dispatch_tile<AK, BKC, false, true>(stream, a, b, C, r, M, N, K, lda, ldb, ldc, ldr, tile); \
+      return dispatch_tile<AK, BKC, false, false>(stream, a, b, C, r, M, N, K, lda, ldb, ldc, ldr, tile);            \
+    }                                                                                            \
+  } while (0)
+  if (a_kc && b_kc) GO(true, true);
+  if (a_kc && !b_kc) GO(true, false);
+  if (!a_kc && !b_kc) GO(false, false);
+  GO(false, true);
+#undef GO
+}
