@@ -1,0 +1,280 @@
+"""Pins the CPU oracle (oracle/ref.py) without the reference: closed forms, textbook
+routines, invariants and autograd/finite differences, each chosen so that a dropped term,
+wrong sign or transposed index fails.  The only reference-held known answers on this path
+(the WSD schedule, src/test/optim/config_test.py:22-33, and the shapes of the sequential
+token generator, src/test/data/utils_test.py) are reproduced literally."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import ref
+
+torch.manual_seed(0)
+D64 = torch.float64
+
+
+def test_rms_norm_closed_form_and_invariants():
+    x = torch.randn(5, 7, 16, dtype=D64)
+    w = torch.randn(16, dtype=D64)
+    y = ref.rms_norm_fwd(x, w, 1e-6)
+    assert torch.allclose(y, F.rms_norm(x, (16,), w, 1e-6), atol=1e-12)
+    y1 = ref.rms_norm_fwd(x, torch.ones(16, dtype=D64), 0.0)
+    assert torch.allclose((y1 * y1).mean(-1), torch.ones(5, 7, dtype=D64), atol=1e-12)
+    assert torch.allclose(ref.rms_norm_fwd(3.7 * x, w, 0.0), ref.rms_norm_fwd(x, w, 0.0), atol=1e-12)
+
+
+def test_rms_norm_bwd_matches_autograd():
+    x = torch.randn(4, 6, 32, dtype=D64, requires_grad=True)
+    w = torch.randn(32, dtype=D64, requires_grad=True)
+    dy = torch.randn(4, 6, 32, dtype=D64)
+    y = F.rms_norm(x, (32,), w, 1e-5)
+    gx, gw = torch.autograd.grad(y, (x, w), dy)
+    dx, dw = ref.rms_norm_bwd(x.detach(), w.detach(), dy, 1e-5)
+    assert torch.allclose(dx, gx, atol=1e-11) and torch.allclose(dw, gw, atol=1e-11)
+    # eps = 0: dx is orthogonal to x
+    dx0, _ = ref.rms_norm_bwd(x.detach(), w.detach(), dy, 0.0)
+    assert (dx0 * x.detach()).sum(-1).abs().max() < 1e-10
+
+
+def test_rope_properties():
+    S, Dh = 24, 16
+    cos, sin = ref.rope_tables(S, Dh, 10000.0, dtype=D64)
+    assert cos.shape == (S, Dh // 2)
+    # closed form of one entry
+    assert abs(cos[5, 3].item() - math.cos(5 * 10000.0 ** (-6 / 16))) < 1e-12
+    x = torch.randn(2, S, 3, Dh, dtype=D64)
+    y = ref.rope_fwd(x, cos, sin)
+    assert torch.allclose(y[:, 0], x[:, 0])  # position 0 is the identity
+    # pairs (j, j + D/2) are rotated: their norm is preserved
+    n_in = x[..., :8] ** 2 + x[..., 8:] ** 2
+    n_out = y[..., :8] ** 2 + y[..., 8:] ** 2
+    assert torch.allclose(n_in, n_out, atol=1e-12)
+    # HF rotate_half convention, written out independently
+    c2 = torch.cat([cos, cos], -1)[None, :, None, :]
+    s2 = torch.cat([sin, sin], -1)[None, :, None, :]
+    rot = torch.cat([-x[..., 8:], x[..., :8]], -1)
+    assert torch.allclose(y, x * c2 + rot * s2, atol=1e-12)
+    # relative-position property
+    q = torch.randn(Dh, dtype=D64)
+    k = torch.randn(Dh, dtype=D64)
+    def at(vec, p):
+        t = torch.zeros(1, S, 1, Dh, dtype=D64); t[0, p, 0] = vec
+        return ref.rope_fwd(t, cos, sin)[0, p, 0]
+    assert abs((at(q, 7) @ at(k, 3)) - (at(q, 14) @ at(k, 10))) < 1e-10
+    # bwd == transpose
+    xg = x.clone().requires_grad_(True)
+    dy = torch.randn_like(x)
+    (gx,) = torch.autograd.grad(ref.rope_fwd(xg, cos, sin), xg, dy)
+    assert torch.allclose(ref.rope_bwd(dy, cos, sin), gx, atol=1e-12)
+
+
+def test_linear_against_bruteforce():
+    x = torch.randn(3, 5, dtype=D64); w = torch.randn(4, 5, dtype=D64); dy = torch.randn(3, 4, dtype=D64)
+    y = ref.linear_fwd(x, w)
+    for i in range(3):
+        for o in range(4):
+            assert abs(y[i, o] - sum(x[i, k] * w[o, k] for k in range(5))) < 1e-12
+    dx, dw = ref.linear_bwd(x, w, dy)
+    xg = x.clone().requires_grad_(True); wg = w.clone().requires_grad_(True)
+    gx, gw = torch.autograd.grad(F.linear(xg, wg), (xg, wg), dy)
+    assert torch.allclose(dx, gx) and torch.allclose(dw, gw)
+
+
+@pytest.mark.parametrize("kind", ["silu", "gelu"])
+def test_glu(kind):
+    g = torch.randn(64, dtype=D64) * 3; u = torch.randn(64, dtype=D64); dh = torch.randn(64, dtype=D64)
+    want = (F.silu(g) if kind == "silu" else F.gelu(g, approximate="tanh")) * u
+    assert torch.allclose(ref.glu_fwd(g, u, kind), want, atol=1e-12)
+    gg = g.clone().requires_grad_(True); ug = u.clone().requires_grad_(True)
+    a = (F.silu(gg) if kind == "silu" else F.gelu(gg, approximate="tanh")) * ug
+    eg, eu = torch.autograd.grad(a, (gg, ug), dh)
+    dg, du = ref.glu_bwd(g, u, dh, kind)
+    assert torch.allclose(dg, eg, atol=1e-11) and torch.allclose(du, eu, atol=1e-11)
+
+
+def _attn_autograd(q, k, v, window, softcap):
+    """Independent formulation (masked softmax via additive -inf bias, GQA by expand)."""
+    B, S, H, Dh = q.shape
+    K = k.shape[2]
+    qh = q.permute(0, 2, 1, 3)
+    kh = k.permute(0, 2, 1, 3)[:, :, None].expand(B, K, H // K, S, Dh).reshape(B, H, S, Dh)
+    vh = v.permute(0, 2, 1, 3)[:, :, None].expand(B, K, H // K, S, Dh).reshape(B, H, S, Dh)
+    s = qh @ kh.transpose(-1, -2) / math.sqrt(Dh)
+    if softcap:
+        s = softcap * torch.tanh(s / softcap)
+    bias = torch.zeros(S, S, dtype=q.dtype)
+    for i in range(S):
+        for j in range(S):
+            if j > i or (window is not None and j < i - window):
+                bias[i, j] = float("-inf")
+    p = torch.softmax(s + bias, -1)
+    return (p @ vh).permute(0, 2, 1, 3)
+
+
+@pytest.mark.parametrize("H,K,window,softcap", [(4, 4, None, 0.0), (4, 2, None, 0.0), (4, 2, 5, 0.0), (4, 1, 3, 7.0), (2, 2, None, 2.5)])
+def test_attention_fwd_bwd(H, K, window, softcap):
+    B, S, Dh = 2, 17, 8
+    q = torch.randn(B, S, H, Dh, dtype=D64, requires_grad=True)
+    k = torch.randn(B, S, K, Dh, dtype=D64, requires_grad=True)
+    v = torch.randn(B, S, K, Dh, dtype=D64, requires_grad=True)
+    do = torch.randn(B, S, H, Dh, dtype=D64)
+    want = _attn_autograd(q, k, v, window, softcap)
+    gq, gk, gv = torch.autograd.grad(want, (q, k, v), do)
+    o, lse = ref.attention_fwd(q.detach(), k.detach(), v.detach(), window=window, softcap=softcap)
+    assert torch.allclose(o, want.detach(), atol=1e-11)
+    assert torch.allclose(o[:, 0], v.detach().repeat_interleave(H // K, 2)[:, 0], atol=1e-12)  # first query sees key 0 only
+    dq, dk, dv = ref.attention_bwd(q.detach(), k.detach(), v.detach(), o, lse, do, window=window, softcap=softcap)
+    assert torch.allclose(dq, gq, atol=1e-10) and torch.allclose(dk, gk, atol=1e-10) and torch.allclose(dv, gv, atol=1e-10)
+
+
+def test_attention_textbook_and_limits():
+    B, S, H, K, Dh = 1, 12, 4, 2, 8
+    q = torch.randn(B, S, H, Dh, dtype=D64); k = torch.randn(B, S, K, Dh, dtype=D64); v = torch.randn(B, S, K, Dh, dtype=D64)
+    o, _ = ref.attention_fwd(q, k, v)
+    want = F.scaled_dot_product_attention(q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3), is_causal=True, enable_gqa=True).permute(0, 2, 1, 3)
+    assert torch.allclose(o, want, atol=1e-11)
+    assert torch.allclose(ref.attention_fwd(q, k, v, window=S - 1)[0], o, atol=1e-12)  # window >= S-1 is full causal
+    assert torch.allclose(ref.attention_fwd(q, k, v, softcap=1e9)[0], o, atol=1e-9)   # cap -> inf is no cap
+    # window w keeps exactly w + 1 keys: with w = 0 every query sees only itself
+    assert torch.allclose(ref.attention_fwd(q, k, v, window=0)[0], v.repeat_interleave(2, 2), atol=1e-12)
+    assert ref.attention_mask(6, 2).sum(1).tolist() == [1, 2, 3, 3, 3, 3]
+
+
+def test_cross_entropy():
+    T, V = 9, 11
+    logits = torch.randn(T, V, dtype=D64)
+    labels = torch.randint(0, V, (T,))
+    labels[2] = -100
+    loss, lse, n = ref.cross_entropy_fwd(logits, labels)
+    assert abs(loss - F.cross_entropy(logits, labels, ignore_index=-100)) < 1e-12
+    from scipy.special import logsumexp
+    assert abs(lse[3].item() - logsumexp(logits[3].numpy())) < 1e-12
+    # reference invariant (src/test/nn/functional_test.py:10-18): an appended ignored row changes nothing
+    l2, _, _ = ref.cross_entropy_fwd(torch.cat([logits, torch.randn(1, V, dtype=D64)]), torch.cat([labels, torch.tensor([-100])]))
+    assert abs(l2 - loss) < 1e-12
+    # uniform logits -> ln V
+    assert abs(ref.cross_entropy_fwd(torch.zeros(4, V, dtype=D64), torch.tensor([0, 1, 2, 3]))[0] - math.log(V)) < 1e-12
+    # bwd vs autograd, rows sum to zero
+    lg = logits.clone().requires_grad_(True)
+    (g,) = torch.autograd.grad(F.cross_entropy(lg, labels, ignore_index=-100), lg)
+    d = ref.cross_entropy_bwd(logits, labels)
+    assert torch.allclose(d, g, atol=1e-12)
+    assert d.sum(-1).abs().max() < 1e-12 and d[2].abs().max() == 0
+
+
+def test_cross_entropy_out_of_range_label_quirk():
+    """label == V (made by the synthetic loader when input == V-1): zero loss, zero grad, but
+    the row still counts in the mean (one_hot gives zeros; `where` is labels != -100)."""
+    V = 3
+    logits = torch.tensor([[0.0, 0.0, 0.0], [1.0, 2.0, 3.0], [5.0, 5.0, 5.0]], dtype=D64)
+    labels = torch.tensor([0, V, -100])
+    loss, _, n = ref.cross_entropy_fwd(logits, labels)
+    assert n == 2 and abs(loss - math.log(3) / 2) < 1e-12   # (ln3 + 0) / 2, hand computed
+    d = ref.cross_entropy_bwd(logits, labels)
+    assert torch.allclose(d[0], torch.tensor([1 / 3 - 1, 1 / 3, 1 / 3], dtype=D64) / 2)
+    assert d[1].abs().max() == 0 and d[2].abs().max() == 0
+
+
+def test_final_softcap_ce_matches_autograd():
+    T, V, c = 6, 13, 3.0
+    logits = torch.randn(T, V, dtype=D64) * 4
+    labels = torch.randint(0, V, (T,))
+    lg = logits.clone().requires_grad_(True)
+    l = F.cross_entropy(c * torch.tanh(lg / c), labels)
+    (g,) = torch.autograd.grad(l, lg)
+    assert abs(ref.cross_entropy_fwd(logits, labels, softcap=c)[0] - l.detach()) < 1e-12
+    assert torch.allclose(ref.cross_entropy_bwd(logits, labels, softcap=c), g, atol=1e-12)
+
+
+def test_adamw_hand_example_and_torch():
+    # 1 element, 2 steps, computed by hand: b1=.9 b2=.999 eps=1e-8 wd=.1 lr=.01, p0=1, g=(0.5, -0.25)
+    p, m, v = torch.tensor([1.0], dtype=D64), torch.zeros(1, dtype=D64), torch.zeros(1, dtype=D64)
+    p, m, v = ref.adamw_step(p, torch.tensor([0.5], dtype=D64), m, v, step=1, lr=0.01, wd=0.1)
+    # step 1: mhat = g, vhat = g^2 -> update = sign(g) (+ wd p)
+    assert abs(p.item() - (1 - 0.01 * (0.5 / (0.5 + 1e-8) + 0.1 * 1.0))) < 1e-15
+    p1 = p.item()
+    p, m, v = ref.adamw_step(p, torch.tensor([-0.25], dtype=D64), m, v, step=2, lr=0.01, wd=0.1)
+    m2 = 0.9 * 0.05 + 0.1 * -0.25; v2 = 0.999 * 0.00025 + 0.001 * 0.0625
+    want = p1 - 0.01 * ((m2 / (1 - 0.81)) / (math.sqrt(v2 / (1 - 0.999 ** 2)) + 1e-8) + 0.1 * p1)
+    assert abs(p.item() - want) < 1e-15
+    # g = 0 -> pure decay
+    p0 = torch.tensor([2.0], dtype=D64)
+    assert abs(ref.adamw_step(p0, torch.zeros(1, dtype=D64), torch.zeros(1, dtype=D64), torch.zeros(1, dtype=D64), step=1, lr=0.1, wd=0.5)[0].item() - 2.0 * (1 - 0.05)) < 1e-15
+    # torch.optim.AdamW is algebraically the same update
+    w = torch.randn(50, dtype=D64)
+    tp = w.clone().requires_grad_(True)
+    opt = torch.optim.AdamW([tp], lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    p, m, v = w.clone(), torch.zeros_like(w), torch.zeros_like(w)
+    for t in range(1, 6):
+        g = torch.randn(50, dtype=D64)
+        tp.grad = g.clone(); opt.step()
+        p, m, v = ref.adamw_step(p, g, m, v, step=t, lr=3e-3, b1=0.9, b2=0.95, wd=0.1)
+    assert torch.allclose(p, tp.detach(), atol=1e-12)
+
+
+def test_schedules_known_answers():
+    # literal values of the reference's own test, src/test/optim/config_test.py:22-33
+    r = [ref.wsd_lr(s, warmup_steps=10, stable_steps=10, decay_steps=10, peak=1.0) for s in range(31)]
+    assert (r[0], r[5], r[10], r[20], r[25], r[30]) == (0.0, 0.5, 1.0, 1.0, 0.5, 0.0)
+    kw = dict(warmup_steps=20, decay_steps=80, peak=1e-4, init=1e-6, end=1e-6)
+    assert ref.warmup_cosine_lr(0, **kw) == 1e-6
+    assert abs(ref.warmup_cosine_lr(20, **kw) - 1e-4) < 1e-18
+    assert abs(ref.warmup_cosine_lr(60, **kw) - (1e-6 + (1e-4 - 1e-6) * 0.5)) < 1e-18
+    assert abs(ref.warmup_cosine_lr(100, **kw) - 1e-6) < 1e-18
+
+
+def test_sequential_tokens():
+    ins, tg = ref.sequential_tokens(torch.tensor([0, 5, 9]), 8, 10)
+    assert ins.shape == (3, 8) and ins.dtype == torch.int32
+    assert ins[1].tolist() == [5, 6, 7, 8, 9, 0, 1, 2]
+    assert tg[1].tolist() == [6, 7, 8, 9, 10, 1, 2, 3]  # target == V after input V-1
+
+
+def test_embedding_scatter_add():
+    ids = torch.tensor([[1, 3, 1]])
+    dh = torch.arange(6, dtype=D64).reshape(1, 3, 2)
+    dw = ref.embed_bwd(ids, dh, 5)
+    assert dw[1].tolist() == [4.0, 6.0] and dw[3].tolist() == [2.0, 3.0] and dw[0].abs().sum() == 0
+
+
+def _autograd_model_loss(cfg, P, ids, labels):
+    """Forward only from the oracle's forward pieces; autograd supplies the gradients."""
+    h = P["embedding.weight"][ids.long()]
+    for l in range(cfg.n_layers):
+        h, _ = ref.block_fwd(cfg, P, l, h)
+    hn = ref.rms_norm_fwd(h, P["norm.weight"], cfg.eps)
+    w = P["embedding.weight"] if cfg.tied else P["lm_head.w_out.weight"]
+    logits = hn @ w.t()
+    return ref.cross_entropy_fwd(logits.reshape(-1, cfg.vocab), labels.reshape(-1), softcap=cfg.final_softcap)[0]
+
+
+@pytest.mark.parametrize("kind", ["pre", "reordered", "gemma"])
+def test_model_grads_match_autograd(kind):
+    cfg = ref.ModelConfig(vocab=37, d_model=16, n_layers=2, n_heads=4, n_kv_heads=2 if kind == "gemma" else 4,
+                          head_dim=4, hidden=24, layer_type=kind, act="gelu" if kind == "gemma" else "silu",
+                          qk_norm=kind != "pre", windows=[3, None] if kind == "gemma" else None,
+                          rope_theta_layers=[1e4, 1e6] if kind == "gemma" else None,
+                          attn_softcap=5.0 if kind == "gemma" else 0.0, final_softcap=3.0 if kind == "gemma" else 0.0,
+                          tied=kind == "gemma")
+    P = {k: (v.double() * (10 if "norm" not in k else 1) + (0.1 * torch.randn_like(v.double()) if "norm" in k else 0)).requires_grad_(True)
+         for k, v in ref.init_params(cfg, seed=1).items()}
+    ids = torch.randint(0, cfg.vocab, (2, 9)); labels = torch.randint(0, cfg.vocab, (2, 9)); labels[0, 2] = -100; labels[1, 1] = cfg.vocab
+    loss = _autograd_model_loss(cfg, P, ids, labels)
+    names = list(P)
+    grads = torch.autograd.grad(loss, [P[n] for n in names])
+    Pd = {k: v.detach() for k, v in P.items()}
+    loss2, G = ref.model_loss_and_grads(cfg, Pd, ids, labels)
+    assert abs(loss2 - loss.detach()) < 1e-12
+    for n, g in zip(names, grads):
+        assert torch.allclose(G[n], g, atol=1e-10, rtol=1e-8), n
+
+
+def test_train_step_decreases_loss_and_masks_decay():
+    cfg = ref.ModelConfig(vocab=50, d_model=16, n_layers=1, n_heads=2, n_kv_heads=2, head_dim=8, hidden=32)
+    master = ref.init_params(cfg, seed=0)
+    opt = {"m": {k: torch.zeros_like(v) for k, v in master.items()}, "v": {k: torch.zeros_like(v) for k, v in master.items()}}
+    ids = torch.randint(0, 50, (2, 8)); labels = torch.randint(0, 50, (2, 8))
+    losses = [ref.train_step(cfg, master, opt, ids, labels, step=s, lr=1e-2, wd=0.1)[0].item() for s in range(1, 6)]
+    assert losses[-1] < losses[0]
