@@ -1,0 +1,742 @@
+// Causal GQA flash attention for gfx950, head_dim 128, BSHD layout, bf16 in/out, fp32
+// softmax statistics, optional sliding window and tanh logit soft-cap.
+//
+// Replaces the cuDNN fused-attention custom call that
+// jax.nn.dot_product_attention(is_causal=True, local_window_size=w) lowers to
+// (reference src/olmax/nn/attention.py:96-103) and its autodiff transpose.
+// Mask: key j visible to query i iff j <= i and (w < 0 or j >= i - w).
+//
+// All three kernels keep the score tile TRANSPOSED in the MFMA accumulators so that each
+// lane owns one query (forward, dQ) or one key (dK/dV) column: row statistics become
+// per-lane scalars, and the exponentiated tile is already laid out as the B operand of the
+// next v_mfma_f32_32x32x16_bf16 (k index = accumulator row pattern).  The operand that must
+// be read against its storage order (V^T, K^T, Q^T, dO^T) comes from LDS through
+// ds_read_b64_tr_b16.  K/V (or Q/dO) tiles are double buffered in LDS with a register-held
+// prefetch of the next tile; 16-byte chunks are XOR-swizzled so that both ds_read_b128 and
+// the transposing reads are bank-conflict free.
+//
+// Backward is split in two deterministic kernels (no atomics): dK/dV with the key tile
+// stationary, dQ with the query tile stationary; each recomputes P from the saved LSE.
+#include "common.h"
+
+extern "C" int32_t olmax_fill_zero(hipStream_t stream, void* p, int64_t nbytes);
+
+namespace {
+
+__device__ __forceinline__ float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+// chunk swizzle: distinct over any 8 consecutive rows (b128 reads) and pair-distinct over
+// any aligned 4 consecutive rows (transposing b64 reads)
+__device__ __forceinline__ int swz(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
+
+// byte offset of 16B chunk `c` (0..15) of row `row` in a [rows][128] bf16 tile
+__device__ __forceinline__ int tile_off(int row, int c) { return row * 256 + ((c ^ swz(row)) << 4); }
+
+// A/B operand fragment with the k index contiguous in storage: row `row`, k-step s (16 wide)
+__device__ __forceinline__ bf16x8 frag_kc(const unsigned char* tile, int row, int s, int lhi) {
+  return *reinterpret_cast<const bf16x8*>(tile + tile_off(row, 2 * s + lhi));
+}
+
+// A operand fragment read transposed: rows of the MFMA = storage columns col0 + (lane % 32),
+// k index = storage rows {r0 + 4*kg + 0..3, r0 + 8 + 4*kg + 0..3}
+__device__ __forceinline__ bf16x8 frag_tr(const unsigned char* tile, int r0, int col0, int lane) {
+  const int j16 = lane & 15, g16 = lane >> 4;
+  const int col = col0 + ((g16 & 1) << 4) + ((j16 & 3) << 2);
+  Pack8 p;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const int row = r0 + ((g16 >> 1) << 2) + (h << 3) + (j16 >> 2);
+    const int off = row * 256 + ((((col >> 3)) ^ swz(row)) << 4) + ((col & 7) << 1);
+    s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(tile + off));
+    p.u[h * 2 + 0] = ((u32x2&)t)[0];
+    p.u[h * 2 + 1] = ((u32x2&)t)[1];
+  }
+  return p.v;
+}
+
+__device__ __forceinline__ bf16x8 pack_bf16x8(const f32x16& a, int base) {
+  bf16x8 r;
+#pragma unroll
+  for (int e = 0; e < 8; e++) r[e] = f2bf(a[base + e]);
+  return r;
+}
+
+__device__ __forceinline__ float fast_tanh(float x) {
+  // tanh(x) = 1 - 2 / (exp(2x) + 1); exact enough in fp32 for |x| up to saturation
+  const float e = __expf(2.f * x);
+  return 1.f - 2.f / (e + 1.f);
+}
+
+// ---------------------------------------------------------------------------------------
+// Forward.  grid = (ceil(S/128), H, B); 256 threads; wave w owns queries i0+32w .. +31.
+// ---------------------------------------------------------------------------------------
+template <bool CAP>
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
+    const bf16* __restrict__ Q, const bf16* __restrict__ K, const bf16* __restrict__ V,
+    bf16* __restrict__ O, float* __restrict__ LSE, int S, int H, int KH, int64_t ldq, int64_t ldk,
+    int64_t ldv, int64_t ldo, float scale, int window, float cap) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [2][K 16K | V 16K]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int qt = gridDim.x - 1 - blockIdx.x;  // longest rows first
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int kh = h / (H / KH);
+  const int i0 = qt * 128;
+  const int iw0 = i0 + wave * 32;  // first query of this wave
+  const int qi = iw0 + l32;        // this lane's query
+  const int qic = min(qi, S - 1);
+
+  bf16x8 qf[8];
+  {
+    const bf16* qp = Q + ((int64_t)b * S + qic) * ldq + h * 128 + lhi * 8;
+#pragma unroll
+    for (int s = 0; s < 8; s++) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
+  }
+  const int j_lo = window >= 0 ? max(0, i0 - window) : 0;
+  const int t_lo = j_lo >> 6;
+  const int t_hi = min(i0 + 127, S - 1) >> 6;  // inclusive
+
+  f32x16 o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[dt][r] = 0.f;
+  float m = -INFINITY, lsum = 0.f;
+
+  // tile loader: 64 rows x 16 chunks for K and V -> 4 + 4 chunks per thread
+  u32x4 kreg[4], vreg[4];
+  const bf16* kbase = K + (int64_t)b * S * ldk + kh * 128;
+  const bf16* vbase = V + (int64_t)b * S * ldv + kh * 128;
+  auto gload = [&](int t) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int q = i * 256 + tid;
+      const int row = q >> 4, c = q & 15;
+      const int j = min(t * 64 + row, S - 1);
+      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)j * ldk + c * 8);
+      vreg[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)j * ldv + c * 8);
+    }
+  };
+  auto lstore = [&](int stage) {
+    unsigned char* sk = smem + stage * 32768;
+    unsigned char* sv = sk + 16384;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int q = i * 256 + tid;
+      const int row = q >> 4, c = q & 15;
+      *reinterpret_cast<u32x4*>(sk + tile_off(row, c)) = kreg[i];
+      *reinterpret_cast<u32x4*>(sv + tile_off(row, c)) = vreg[i];
+    }
+  };
+  const float sc2 = scale * LOG2E;
+
+  gload(t_lo);
+  lstore(0);
+  __syncthreads();
+  for (int t = t_lo; t <= t_hi; t++) {
+    const int cur = (t - t_lo) & 1;
+    if (t < t_hi) gload(t + 1);
+    const int j0 = t * 64;
+    // skip tiles this wave cannot see at all
+    const bool visible = (j0 <= iw0 + 31) && (window < 0 || j0 + 63 >= iw0 - window);
+    if (visible) {
+      const unsigned char* sk = smem + cur * 32768;
+      const unsigned char* sv = sk + 16384;
+      f32x16 st[2];
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) st[jt][r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+          st[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sk, jt * 32 + l32, s, lhi), qf[s], st[jt], 0, 0, 0);
+      }
+      const bool need_mask = (j0 + 63 > iw0) || (window >= 0 && j0 < iw0 + 31 - window);
+      float mt = -INFINITY;
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float s = st[jt][r];
+          if (CAP) s = cap * fast_tanh(s * scale / cap) * LOG2E;
+          else s = s * sc2;
+          if (need_mask) {
+            const int j = j0 + jt * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
+            const bool ok = (j <= qi) && (window < 0 || j >= qi - window);
+            s = ok ? s : -INFINITY;
+          }
+          st[jt][r] = s;
+          mt = fmaxf(mt, s);
+        }
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float m_new = fmaxf(m, mt);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = fexp2(m - m_use);  // m = -inf -> 0
+      float ps = 0.f;
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float p = fexp2(st[jt][r] - m_use);
+          st[jt][r] = p;
+          ps += p;
+        }
+      lsum = lsum * alpha + ps;
+      m = m_new;
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+      bf16x8 pb[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) pb[u] = pack_bf16x8(st[u >> 1], (u & 1) * 8);
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(sv, u * 16, dt * 32, lane), pb[u], o[dt], 0, 0, 0);
+    }
+    if (t < t_hi) lstore(cur ^ 1);
+    __syncthreads();
+  }
+  const float ltot = lsum + __shfl_xor(lsum, 32, 64);
+  const float inv = ltot > 0.f ? 1.f / ltot : 0.f;
+  if (qi < S) {
+    bf16* op = O + ((int64_t)b * S + qi) * ldo + h * 128;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        Pack4 pk;
+#pragma unroll
+        for (int e = 0; e < 4; e++) pk.e[e] = f2bf(o[dt][g * 4 + e] * inv);
+        *reinterpret_cast<u32x2*>(op + dt * 32 + g * 8 + lhi * 4) = pk.u;
+      }
+    if (lhi == 0) LSE[((int64_t)b * H + h) * S + qi] = (m + log2f(ltot)) * LN2;
+  }
+}
+
+// delta[b,h,i] = sum_d dO[i,h,d] * O[i,h,d]; one 16-lane group per (token, head)
+__global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict__ O,
+                                                         const bf16* __restrict__ dO,
+                                                         float* __restrict__ delta, int B, int S, int H,
+                                                         int64_t ldo, int64_t lddo) {
+  const int sub = threadIdx.x & 15;
+  const int64_t unit = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+  if (unit >= (int64_t)B * S * H) return;
+  const int64_t tok = unit / H;
+  const int h = (int)(unit % H);
+  Pack8 a, c;
+  a.u = *reinterpret_cast<const u32x4*>(O + tok * ldo + h * 128 + sub * 8);
+  c.u = *reinterpret_cast<const u32x4*>(dO + tok * lddo + h * 128 + sub * 8);
+  float s = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) s += bf2f(a.e[e]) * bf2f(c.e[e]);
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+  if (sub == 0) {
+    const int64_t bb = tok / S, i = tok % S;
+    delta[(bb * H + h) * S + i] = s;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// dQ.  Same tiling as the forward: grid = (ceil(S/128), H, B); K/V tiles stream through LDS.
+// ---------------------------------------------------------------------------------------
+template <bool CAP>
+__global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(
+    const bf16* __restrict__ Q, const bf16* __restrict__ K, const bf16* __restrict__ V,
+    const bf16* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ DELTA,
+    bf16* __restrict__ dQ, int S, int H, int KH, int64_t ldq, int64_t ldk, int64_t ldv, int64_t lddo,
+    int64_t lddq, float scale, int window, float cap) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int qt = gridDim.x - 1 - blockIdx.x;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int kh = h / (H / KH);
+  const int i0 = qt * 128;
+  const int iw0 = i0 + wave * 32;
+  const int qi = iw0 + l32;
+  const int qic = min(qi, S - 1);
+
+  bf16x8 qf[8], dof[8];
+  {
+    const bf16* qp = Q + ((int64_t)b * S + qic) * ldq + h * 128 + lhi * 8;
+    const bf16* dp = dO + ((int64_t)b * S + qic) * lddo + h * 128 + lhi * 8;
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+      qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
+      dof[s] = *reinterpret_cast<const bf16x8*>(dp + s * 16);
+    }
+  }
+  const float lse2 = LSE[((int64_t)b * H + h) * S + qic] * LOG2E;
+  const float dlt = DELTA[((int64_t)b * H + h) * S + qic];
+  const int j_lo = window >= 0 ? max(0, i0 - window) : 0;
+  const int t_lo = j_lo >> 6;
+  const int t_hi = min(i0 + 127, S - 1) >> 6;
+
+  f32x16 dq[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dq[dt][r] = 0.f;
+
+  u32x4 kreg[4], vreg[4];
+  const bf16* kbase = K + (int64_t)b * S * ldk + kh * 128;
+  const bf16* vbase = V + (int64_t)b * S * ldv + kh * 128;
+  auto gload = [&](int t) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int q = i * 256 + tid;
+      const int row = q >> 4, c = q & 15;
+      const int j = min(t * 64 + row, S - 1);
+      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)j * ldk + c * 8);
+      vreg[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)j * ldv + c * 8);
+    }
+  };
+  auto lstore = [&](int stage) {
+    unsigned char* sk = smem + stage * 32768;
+    unsigned char* sv = sk + 16384;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int q = i * 256 + tid;
+      const int row = q >> 4, c = q & 15;
+      *reinterpret_cast<u32x4*>(sk + tile_off(row, c)) = kreg[i];
+      *reinterpret_cast<u32x4*>(sv + tile_off(row, c)) = vreg[i];
+    }
+  };
+  const float sc2 = scale * LOG2E;
+
+  gload(t_lo);
+  lstore(0);
+  __syncthreads();
+  for (int t = t_lo; t <= t_hi; t++) {
+    const int cur = (t - t_lo) & 1;
+    if (t < t_hi) gload(t + 1);
+    const int j0 = t * 64;
+    const bool visible = (j0 <= iw0 + 31) && (window < 0 || j0 + 63 >= iw0 - window);
+    if (visible) {
+      const unsigned char* sk = smem + cur * 32768;
+      const unsigned char* sv = sk + 16384;
+      f32x16 st[2], dpt[2];
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) { st[jt][r] = 0.f; dpt[jt][r] = 0.f; }
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+          st[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sk, jt * 32 + l32, s, lhi), qf[s], st[jt], 0, 0, 0);
+          dpt[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sv, jt * 32 + l32, s, lhi), dof[s], dpt[jt], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float s = st[jt][r], chain = 1.f;
+          if (CAP) {
+            const float th = fast_tanh(s * scale / cap);
+            s = cap * th * LOG2E;
+            chain = 1.f - th * th;
+          } else {
+            s = s * sc2;
+          }
+          const int j = j0 + jt * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
+          const bool ok = (j <= qi) && (window < 0 || j >= qi - window);
+          const float p = ok ? fexp2(s - lse2) : 0.f;
+          st[jt][r] = p * (dpt[jt][r] - dlt) * chain;
+        }
+      bf16x8 dsb[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) dsb[u] = pack_bf16x8(st[u >> 1], (u & 1) * 8);
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+          dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(sk, u * 16, dt * 32, lane), dsb[u], dq[dt], 0, 0, 0);
+    }
+    if (t < t_hi) lstore(cur ^ 1);
+    __syncthreads();
+  }
+  if (qi < S) {
+    bf16* op = dQ + ((int64_t)b * S + qi) * lddq + h * 128;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        Pack4 pk;
+#pragma unroll
+        for (int e = 0; e < 4; e++) pk.e[e] = f2bf(dq[dt][g * 4 + e] * scale);
+        *reinterpret_cast<u32x2*>(op + dt * 32 + g * 8 + lhi * 4) = pk.u;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// dK/dV.  grid = (ceil(S/128), KH, B); wave w owns keys j0+32w..+31; loops over the query
+// heads of its group and over 64-row Q/dO tiles from the diagonal downwards.
+// LDS per stage: Q 16K | dO 16K | lse 256 B | delta 256 B
+// ---------------------------------------------------------------------------------------
+template <bool CAP>
+__global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(
+    const bf16* __restrict__ Q, const bf16* __restrict__ K, const bf16* __restrict__ V,
+    const bf16* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ DELTA,
+    bf16* __restrict__ dK, bf16* __restrict__ dV, int S, int H, int KH, int64_t ldq, int64_t ldk,
+    int64_t ldv, int64_t lddo, int64_t lddk, int64_t lddv, float scale, int window, float cap) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int STAGE = 32768 + 512;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int kt = blockIdx.x;
+  const int kh = blockIdx.y, b = blockIdx.z;
+  const int rep = H / KH;
+  const int j0 = kt * 128;
+  const int jw0 = j0 + wave * 32;
+  const int kj = jw0 + l32;  // this lane's key
+  const int kjc = min(kj, S - 1);
+
+  bf16x8 kf[8], vf[8];
+  {
+    const bf16* kp = K + ((int64_t)b * S + kjc) * ldk + kh * 128 + lhi * 8;
+    const bf16* vp = V + ((int64_t)b * S + kjc) * ldv + kh * 128 + lhi * 8;
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+      kf[s] = *reinterpret_cast<const bf16x8*>(kp + s * 16);
+      vf[s] = *reinterpret_cast<const bf16x8*>(vp + s * 16);
+    }
+  }
+  f32x16 dk[4], dv[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) { dk[dt][r] = 0.f; dv[dt][r] = 0.f; }
+
+  const int i_hi = window >= 0 ? min(S - 1, j0 + 127 + window) : S - 1;
+  const int t_lo = j0 >> 6;
+  const int t_hi = i_hi >> 6;  // inclusive, 64-row query tiles
+  const int ntile = t_hi - t_lo + 1;
+  const int total = ntile * rep;  // flattened (head, tile) iteration space
+  const float sc2 = scale * LOG2E;
+
+  u32x4 qreg[4], oreg[4];
+  float sreg = 0.f;
+  auto gload = [&](int it) {
+    const int hq = kh * rep + it / ntile;
+    const int t = t_lo + it % ntile;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int q = i * 256 + tid;
+      const int row = q >> 4, c = q & 15;
+      const int ii = min(t * 64 + row, S - 1);
+      qreg[i] = *reinterpret_cast<const u32x4*>(Q + ((int64_t)b * S + ii) * ldq + hq * 128 + c * 8);
+      oreg[i] = *reinterpret_cast<const u32x4*>(dO + ((int64_t)b * S + ii) * lddo + hq * 128 + c * 8);
+    }
+    if (tid < 128) {
+      const int ii = min(t * 64 + (tid & 63), S - 1);
+      const float* src = tid < 64 ? LSE : DELTA;
+      sreg = src[((int64_t)b * H + hq) * S + ii];
+      if (tid < 64) sreg *= LOG2E;
+    }
+  };
+  auto lstore = [&](int stage) {
+    unsigned char* sq = smem + stage * STAGE;
+    unsigned char* so = sq + 16384;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int q = i * 256 + tid;
+      const int row = q >> 4, c = q & 15;
+      *reinterpret_cast<u32x4*>(sq + tile_off(row, c)) = qreg[i];
+      *reinterpret_cast<u32x4*>(so + tile_off(row, c)) = oreg[i];
+    }
+    if (tid < 128) reinterpret_cast<float*>(sq + 32768)[tid] = sreg;
+  };
+
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  for (int it = 0; it < total; it++) {
+    const int cur = it & 1;
+    if (it + 1 < total) gload(it + 1);
+    const int t = t_lo + it % ntile;
+    const int ib = t * 64;  // first query of the tile
+    // this wave sees the tile iff some i in [ib, ib+63] has j <= i <= j + window for its keys
+    const bool visible = (ib + 63 >= jw0) && (window < 0 || ib <= jw0 + 31 + window);
+    if (visible) {
+      const unsigned char* sq = smem + cur * STAGE;
+      const unsigned char* so = sq + 16384;
+      const float* slse = reinterpret_cast<const float*>(sq + 32768);
+      const float* sdel = slse + 64;
+      f32x16 sa[2], dpa[2];
+#pragma unroll
+      for (int itl = 0; itl < 2; itl++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) { sa[itl][r] = 0.f; dpa[itl][r] = 0.f; }
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+          sa[itl] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sq, itl * 32 + l32, s, lhi), kf[s], sa[itl], 0, 0, 0);
+          dpa[itl] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(so, itl * 32 + l32, s, lhi), vf[s], dpa[itl], 0, 0, 0);
+        }
+      }
+      // accumulator rows are queries i = ib + 32*itl + 8*(r/4) + 4*lhi + r%4; column = key kj
+#pragma unroll
+      for (int itl = 0; itl < 2; itl++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const int il = itl * 32 + g * 8 + lhi * 4;
+          const f32x4 l4 = *reinterpret_cast<const f32x4*>(slse + il);
+          const f32x4 d4 = *reinterpret_cast<const f32x4*>(sdel + il);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int r = g * 4 + e;
+            const int i = ib + il + e;
+            float s = sa[itl][r], chain = 1.f;
+            if (CAP) {
+              const float th = fast_tanh(s * scale / cap);
+              s = cap * th * LOG2E;
+              chain = 1.f - th * th;
+            } else {
+              s = s * sc2;
+            }
+            const bool ok = (kj <= i) && (i < S) && (window < 0 || kj >= i - window);
+            const float p = ok ? fexp2(s - l4[e]) : 0.f;
+            sa[itl][r] = p;
+            dpa[itl][r] = p * (dpa[itl][r] - d4[e]) * chain;
+          }
+        }
+      bf16x8 pb[4], dsb[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        pb[u] = pack_bf16x8(sa[u >> 1], (u & 1) * 8);
+        dsb[u] = pack_bf16x8(dpa[u >> 1], (u & 1) * 8);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+          dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(so, u * 16, dt * 32, lane), pb[u], dv[dt], 0, 0, 0);
+          dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(sq, u * 16, dt * 32, lane), dsb[u], dk[dt], 0, 0, 0);
+        }
+    }
+    if (it + 1 < total) lstore(cur ^ 1);
+    __syncthreads();
+  }
+  if (kj < S) {
+    bf16* kp = dK + ((int64_t)b * S + kj) * lddk + kh * 128;
+    bf16* vp = dV + ((int64_t)b * S + kj) * lddv + kh * 128;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        Pack4 pk, pv;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          pk.e[e] = f2bf(dk[dt][g * 4 + e] * scale);
+          pv.e[e] = f2bf(dv[dt][g * 4 + e]);
+        }
+        *reinterpret_cast<u32x2*>(kp + dt * 32 + g * 8 + lhi * 4) = pk.u;
+        *reinterpret_cast<u32x2*>(vp + dt * 32 + g * 8 + lhi * 4) = pv.u;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Any head_dim (<= 256): one wave per (batch, head, query); scores staged in LDS.
+// Used by the small shapes of unit tests and the CPU-sized reference configuration.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void attn_fwd_generic(
+    const bf16* __restrict__ Q, const bf16* __restrict__ K, const bf16* __restrict__ V,
+    bf16* __restrict__ O, float* __restrict__ LSE, int S, int H, int KH, int D, int64_t ldq,
+    int64_t ldk, int64_t ldv, int64_t ldo, float scale, int window, float cap) {
+  extern __shared__ float sc[];  // S floats
+  const int i = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int kh = h / (H / KH);
+  const int lane = threadIdx.x;
+  const bf16* q = Q + ((int64_t)b * S + i) * ldq + h * D;
+  const int lo = window >= 0 ? max(0, i - window) : 0;
+  float mx = -INFINITY;
+  for (int j = lo + lane; j <= i; j += 64) {
+    const bf16* k = K + ((int64_t)b * S + j) * ldk + kh * D;
+    float s = 0.f;
+    for (int d = 0; d < D; d++) s += bf2f(q[d]) * bf2f(k[d]);
+    s *= scale;
+    if (cap > 0.f) s = cap * tanhf(s / cap);
+    sc[j] = s;
+    mx = fmaxf(mx, s);
+  }
+  mx = wave_max(mx);
+  float sm = 0.f;
+  for (int j = lo + lane; j <= i; j += 64) sm += __expf(sc[j] - mx);
+  sm = wave_sum(sm);
+  const float lse = mx + __logf(sm);
+  __syncthreads();
+  for (int d = lane; d < D; d += 64) {
+    float acc = 0.f;
+    for (int j = lo; j <= i; j++) {
+      const float p = bf2f(f2bf(__expf(sc[j] - lse)));
+      acc += p * bf2f(V[((int64_t)b * S + j) * ldv + kh * D + d]);
+    }
+    O[((int64_t)b * S + i) * ldo + h * D + d] = f2bf(acc);
+  }
+  if (lane == 0) LSE[((int64_t)b * H + h) * S + i] = lse;
+}
+
+// dQ directly; dK/dV accumulated with fp32 atomics into [B*S, KH*D] workspaces.
+__global__ __launch_bounds__(64) void attn_bwd_generic(
+    const bf16* __restrict__ Q, const bf16* __restrict__ K, const bf16* __restrict__ V,
+    const bf16* __restrict__ O, const bf16* __restrict__ dO, const float* __restrict__ LSE,
+    bf16* __restrict__ dQ, float* __restrict__ dKf, float* __restrict__ dVf, int S, int H, int KH,
+    int D, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo, int64_t lddq,
+    float scale, int window, float cap) {
+  extern __shared__ float sh[];  // p[S], ds[S]
+  float* sp = sh;
+  float* sds = sh + S;
+  const int i = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int kh = h / (H / KH);
+  const int lane = threadIdx.x;
+  const bf16* q = Q + ((int64_t)b * S + i) * ldq + h * D;
+  const bf16* o = O + ((int64_t)b * S + i) * ldo + h * D;
+  const bf16* go = dO + ((int64_t)b * S + i) * lddo + h * D;
+  const float lse = LSE[((int64_t)b * H + h) * S + i];
+  const int lo = window >= 0 ? max(0, i - window) : 0;
+  float dl = 0.f;
+  for (int d = lane; d < D; d += 64) dl += bf2f(o[d]) * bf2f(go[d]);
+  dl = wave_sum(dl);
+  for (int j = lo + lane; j <= i; j += 64) {
+    const bf16* k = K + ((int64_t)b * S + j) * ldk + kh * D;
+    const bf16* v = V + ((int64_t)b * S + j) * ldv + kh * D;
+    float s = 0.f, dp = 0.f;
+    for (int d = 0; d < D; d++) {
+      s += bf2f(q[d]) * bf2f(k[d]);
+      dp += bf2f(go[d]) * bf2f(v[d]);
+    }
+    s *= scale;
+    float chain = 1.f;
+    if (cap > 0.f) {
+      const float th = tanhf(s / cap);
+      s = cap * th;
+      chain = 1.f - th * th;
+    }
+    const float p = __expf(s - lse);
+    sp[j] = bf2f(f2bf(p));
+    sds[j] = bf2f(f2bf(p * (dp - dl) * chain));
+  }
+  __syncthreads();
+  for (int d = lane; d < D; d += 64) {
+    float acc = 0.f;
+    const float qd = bf2f(q[d]), god = bf2f(go[d]);
+    for (int j = lo; j <= i; j++) {
+      acc += sds[j] * bf2f(K[((int64_t)b * S + j) * ldk + kh * D + d]);
+      atomicAdd(&dKf[((int64_t)b * S + j) * KH * D + kh * D + d], sds[j] * qd * scale);
+      atomicAdd(&dVf[((int64_t)b * S + j) * KH * D + kh * D + d], sp[j] * god);
+    }
+    dQ[((int64_t)b * S + i) * lddq + h * D + d] = f2bf(acc * scale);
+  }
+}
+
+__global__ void strided_cast_f32_bf16(const float* __restrict__ in, bf16* __restrict__ out,
+                                      int64_t rows, int cols, int64_t ldo) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * cols) return;
+  out[(i / cols) * ldo + i % cols] = f2bf(in[i]);
+}
+
+bool fast_ok(int D, const void* q, const void* k, const void* v, const void* o, int64_t ldq,
+             int64_t ldk, int64_t ldv, int64_t ldo) {
+  return D == 128 && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) && ldq % 8 == 0 &&
+         ldk % 8 == 0 && ldv % 8 == 0 && ldo % 8 == 0;
+}
+
+}  // namespace
+
+// q [B*S, ldq] (head h at columns h*D..), k/v [B*S, ldk/ldv] (KH heads), o [B*S, ldo],
+// lse [B, H, S] fp32 (natural log of the masked softmax normaliser of the scaled, capped scores).
+// window < 0: global causal; window >= 0: keys i-window..i.  softcap <= 0: off.
+extern "C" int32_t olmax_attn_fwd(hipStream_t stream, const void* q, const void* k, const void* v,
+                                  void* o, float* lse, int32_t B, int32_t S, int32_t H, int32_t KH,
+                                  int32_t D, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo,
+                                  int32_t window, float softcap) {
+  OLMAX_CHECK(q && k && v && o && lse, OLMAX_ERR_ARG, "olmax_attn_fwd: null pointer");
+  OLMAX_CHECK(B > 0 && S > 0 && H > 0 && KH > 0 && D > 0 && H % KH == 0, OLMAX_ERR_SHAPE, "olmax_attn_fwd: bad shape B=%d S=%d H=%d KH=%d D=%d", B, S, H, KH, D);
+  OLMAX_CHECK(ldq >= (int64_t)H * D && ldo >= (int64_t)H * D && ldk >= (int64_t)KH * D && ldv >= (int64_t)KH * D, OLMAX_ERR_SHAPE, "olmax_attn_fwd: row stride smaller than heads*head_dim");
+  const float scale = 1.f / sqrtf((float)D);
+  const bf16 *qp = (const bf16*)q, *kp = (const bf16*)k, *vp = (const bf16*)v;
+  if (fast_ok(D, q, k, v, o, ldq, ldk, ldv, ldo)) {
+    dim3 grid((S + 127) / 128, H, B);
+    if (softcap > 0.f) {
+      static bool set = false;
+      if (!set) { (void)hipFuncSetAttribute((const void*)attn_fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536); set = true; }
+      hipLaunchKernelGGL(attn_fwd_kernel<true>, grid, dim3(256), 65536, stream, qp, kp, vp, (bf16*)o, lse, S, H, KH, ldq, ldk, ldv, ldo, scale, window, softcap);
+    } else {
+      static bool set = false;
+      if (!set) { (void)hipFuncSetAttribute((const void*)attn_fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536); set = true; }
+      hipLaunchKernelGGL(attn_fwd_kernel<false>, grid, dim3(256), 65536, stream, qp, kp, vp, (bf16*)o, lse, S, H, KH, ldq, ldk, ldv, ldo, scale, window, softcap);
+    }
+  } else {
+    OLMAX_CHECK(D <= 256 && (size_t)S * 4 <= 65536, OLMAX_ERR_SHAPE, "olmax_attn_fwd: generic path supports head_dim <= 256 and seq_len <= 16384");
+    hipLaunchKernelGGL(attn_fwd_generic, dim3(S, H, B), dim3(64), (size_t)S * 4, stream, qp, kp, vp, (bf16*)o, lse, S, H, KH, D, ldq, ldk, ldv, ldo, scale, window, softcap);
+  }
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+// Workspace: delta [B,H,S] fp32; the generic (head_dim != 128) path additionally needs two
+// fp32 [B*S, KH*D] accumulators.
+extern "C" int64_t olmax_attn_bwd_workspace_bytes(int32_t B, int32_t S, int32_t H, int32_t KH, int32_t D) {
+  int64_t n = ((int64_t)B * H * S * 4 + 255) / 256 * 256;
+  if (D != 128) n += 2 * (((int64_t)B * S * KH * D * 4 + 255) / 256 * 256);
+  return n;
+}
+
+extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void* k, const void* v,
+                                  const void* o, const float* lse, const void* d_o, void* dq, void* dk,
+                                  void* dv, void* workspace, int64_t workspace_bytes, int32_t B,
+                                  int32_t S, int32_t H, int32_t KH, int32_t D, int64_t ldq, int64_t ldk,
+                                  int64_t ldv, int64_t ldo, int64_t lddo, int64_t lddq, int64_t lddk,
+                                  int64_t lddv, int32_t window, float softcap) {
+  OLMAX_CHECK(q && k && v && o && lse && d_o && dq && dk && dv && workspace, OLMAX_ERR_ARG, "olmax_attn_bwd: null pointer");
+  OLMAX_CHECK(B > 0 && S > 0 && H > 0 && KH > 0 && D > 0 && H % KH == 0, OLMAX_ERR_SHAPE, "olmax_attn_bwd: bad shape");
+  OLMAX_CHECK(workspace_bytes >= olmax_attn_bwd_workspace_bytes(B, S, H, KH, D) && (((uintptr_t)workspace) & 255) == 0, OLMAX_ERR_WORKSPACE, "olmax_attn_bwd: workspace too small or not 256-byte aligned");
+  OLMAX_CHECK(ldq >= (int64_t)H * D && ldo >= (int64_t)H * D && lddo >= (int64_t)H * D && lddq >= (int64_t)H * D && ldk >= (int64_t)KH * D && ldv >= (int64_t)KH * D && lddk >= (int64_t)KH * D && lddv >= (int64_t)KH * D, OLMAX_ERR_SHAPE, "olmax_attn_bwd: row stride smaller than heads*head_dim");
+  const float scale = 1.f / sqrtf((float)D);
+  const bf16 *qp = (const bf16*)q, *kp = (const bf16*)k, *vp = (const bf16*)v, *op = (const bf16*)o, *gop = (const bf16*)d_o;
+  float* delta = (float*)workspace;
+  const bool fast = fast_ok(D, q, k, v, o, ldq, ldk, ldv, ldo) && aligned16(d_o) && aligned16(dq) && aligned16(dk) && aligned16(dv) &&
+                    lddo % 8 == 0 && lddq % 8 == 0 && lddk % 8 == 0 && lddv % 8 == 0;
+  if (fast) {
+    const int64_t units = (int64_t)B * S * H;
+    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((units + 15) / 16)), dim3(256), 0, stream, op, gop, delta, B, S, H, ldo, lddo);
+    dim3 gkv((S + 127) / 128, KH, B), gq((S + 127) / 128, H, B);
+    constexpr int SM_KV = 2 * (32768 + 512);
+    static bool set = false;
+    if (!set) {
+      (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
+      (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
+      (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+      (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+      set = true;
+    }
+    if (softcap > 0.f) {
+      hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, gkv, dim3(256), SM_KV, stream, qp, kp, vp, gop, lse, delta, (bf16*)dk, (bf16*)dv, S, H, KH, ldq, ldk, ldv, lddo, lddk, lddv, scale, window, softcap);
+      hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, gq, dim3(256), 65536, stream, qp, kp, vp, gop, lse, delta, (bf16*)dq, S, H, KH, ldq, ldk, ldv, lddo, lddq, scale, window, softcap);
+    } else {
+      hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, gkv, dim3(256), SM_KV, stream, qp, kp, vp, gop, lse, delta, (bf16*)dk, (bf16*)dv, S, H, KH, ldq, ldk, ldv, lddo, lddk, lddv, scale, window, softcap);
+      hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, gq, dim3(256), 65536, stream, qp, kp, vp, gop, lse, delta, (bf16*)dq, S, H, KH, ldq, ldk, ldv, lddo, lddq, scale, window, softcap);
+    }
+  } else {
+    OLMAX_CHECK(D <= 256 && (size_t)S * 8 <= 65536, OLMAX_ERR_SHAPE, "olmax_attn_bwd: generic path supports head_dim <= 256 and seq_len <= 8192");
+    const int64_t accb = ((int64_t)B * S * KH * D * 4 + 255) / 256 * 256;
+    float* dkf = (float*)((char*)workspace + ((int64_t)B * H * S * 4 + 255) / 256 * 256);
+    float* dvf = (float*)((char*)dkf + accb);
+    { int rc = olmax_fill_zero(stream, dkf, 2 * accb); if (rc) return rc; }
+    hipLaunchKernelGGL(attn_bwd_generic, dim3(S, H, B), dim3(64), (size_t)S * 8, stream, qp, kp, vp, op, gop, lse, (bf16*)dq, dkf, dvf, S, H, KH, D, ldq, ldk, ldv, ldo, lddo, lddq, scale, window, softcap);
+    const int64_t n = (int64_t)B * S * KH * D;
+    hipLaunchKernelGGL(strided_cast_f32_bf16, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, dkf, (bf16*)dk, (int64_t)B * S, KH * D, lddk);
+    hipLaunchKernelGGL(strided_cast_f32_bf16, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, dvf, (bf16*)dv, (int64_t)B * S, KH * D, lddv);
+  }
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}

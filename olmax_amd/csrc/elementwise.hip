@@ -1,0 +1,375 @@
+// HBM-bound elementwise / gather kernels: gated-MLP activation, embedding gather and
+// scatter-add, fused fp32 AdamW (with the bf16 working-copy write), utility fills/casts.
+// 128-bit accesses, grid-stride loops.
+//
+// Reference semantics:
+//   GatedMLP      src/olmax/nn/mlp.py:69-73 (act = jax.nn.silu; jax.nn.gelu(tanh) for Gemma,
+//                 src/olmax/nn/transformer/layer.py:133)
+//   Embedding     src/olmax/nn/embedding.py:30-32
+//   AdamW         optax.adamw configured at src/olmax/optim/config.py:136-156, applied at
+//                 src/olmax/train/trainer.py:745-752; the bf16 copy replaces the per-step
+//                 cast_tree(params, bf16) of src/olmax/train/trainer.py:728
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float act_silu(float g) { return g / (1.f + __expf(-g)); }
+__device__ __forceinline__ float act_silu_grad(float g) {
+  const float s = 1.f / (1.f + __expf(-g));
+  return s * (1.f + g * (1.f - s));
+}
+constexpr float GELU_C = 0.7978845608028654f;  // sqrt(2/pi)
+__device__ __forceinline__ float act_gelu(float g) {
+  return 0.5f * g * (1.f + tanhf(GELU_C * (g + 0.044715f * g * g * g)));
+}
+__device__ __forceinline__ float act_gelu_grad(float g) {
+  const float t = tanhf(GELU_C * (g + 0.044715f * g * g * g));
+  return 0.5f * (1.f + t) + 0.5f * g * (1.f - t * t) * GELU_C * (1.f + 3.f * 0.044715f * g * g);
+}
+
+// gate/up are column blocks of one [T, ld] buffer (or separate buffers); out [T, F].
+template <bool GELU>
+__global__ __launch_bounds__(256) void glu_fwd_kernel(const bf16* __restrict__ gate,
+                                                      const bf16* __restrict__ up,
+                                                      bf16* __restrict__ out, int64_t T, int F,
+                                                      int64_t ldg, int64_t ldu, int64_t ldo) {
+  const int cpr = F / 8;
+  const int64_t total = T * cpr;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t t = i / cpr;
+    const int c = (int)(i % cpr) * 8;
+    Pack8 g, u, o;
+    g.u = *reinterpret_cast<const u32x4*>(gate + t * ldg + c);
+    u.u = *reinterpret_cast<const u32x4*>(up + t * ldu + c);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float gf = bf2f(g.e[e]);
+      const float a = bf2f(f2bf(GELU ? act_gelu(gf) : act_silu(gf)));  // act output is a bf16 array
+      o.e[e] = f2bf(a * bf2f(u.e[e]));
+    }
+    *reinterpret_cast<u32x4*>(out + t * ldo + c) = o.u;
+  }
+}
+
+template <bool GELU>
+__global__ __launch_bounds__(256) void glu_bwd_kernel(const bf16* __restrict__ gate,
+                                                      const bf16* __restrict__ up,
+                                                      const bf16* __restrict__ dh,
+                                                      bf16* __restrict__ dgate,
+                                                      bf16* __restrict__ dup, int64_t T, int F,
+                                                      int64_t ldg, int64_t ldu, int64_t lddh,
+                                                      int64_t lddg, int64_t lddu) {
+  const int cpr = F / 8;
+  const int64_t total = T * cpr;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t t = i / cpr;
+    const int c = (int)(i % cpr) * 8;
+    Pack8 g, u, d, og, ou;
+    g.u = *reinterpret_cast<const u32x4*>(gate + t * ldg + c);
+    u.u = *reinterpret_cast<const u32x4*>(up + t * ldu + c);
+    d.u = *reinterpret_cast<const u32x4*>(dh + t * lddh + c);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float gf = bf2f(g.e[e]), uf = bf2f(u.e[e]), df = bf2f(d.e[e]);
+      og.e[e] = f2bf(df * uf * (GELU ? act_gelu_grad(gf) : act_silu_grad(gf)));
+      ou.e[e] = f2bf(df * (GELU ? act_gelu(gf) : act_silu(gf)));
+    }
+    *reinterpret_cast<u32x4*>(dgate + t * lddg + c) = og.u;
+    *reinterpret_cast<u32x4*>(dup + t * lddu + c) = ou.u;
+  }
+}
+
+template <bool GELU>
+__global__ void glu_fwd_scalar(const bf16* gate, const bf16* up, bf16* out, int64_t T, int F,
+                               int64_t ldg, int64_t ldu, int64_t ldo) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= T * F) return;
+  const int64_t t = i / F;
+  const int c = (int)(i % F);
+  const float gf = bf2f(gate[t * ldg + c]);
+  const float a = bf2f(f2bf(GELU ? act_gelu(gf) : act_silu(gf)));
+  out[t * ldo + c] = f2bf(a * bf2f(up[t * ldu + c]));
+}
+template <bool GELU>
+__global__ void glu_bwd_scalar(const bf16* gate, const bf16* up, const bf16* dh, bf16* dgate,
+                               bf16* dup, int64_t T, int F, int64_t ldg, int64_t ldu, int64_t lddh,
+                               int64_t lddg, int64_t lddu) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= T * F) return;
+  const int64_t t = i / F;
+  const int c = (int)(i % F);
+  const float gf = bf2f(gate[t * ldg + c]), uf = bf2f(up[t * ldu + c]), df = bf2f(dh[t * lddh + c]);
+  dgate[t * lddg + c] = f2bf(df * uf * (GELU ? act_gelu_grad(gf) : act_silu_grad(gf)));
+  dup[t * lddu + c] = f2bf(df * (GELU ? act_gelu(gf) : act_silu(gf)));
+}
+
+// ------------------------------------------------------------------ embedding
+// ids outside [0, V) are clamped (memory safety; the data path never produces them).
+__global__ __launch_bounds__(256) void embed_fwd_kernel(const int32_t* __restrict__ ids,
+                                                        const bf16* __restrict__ W,
+                                                        bf16* __restrict__ out, int64_t T, int d,
+                                                        int V) {
+  const int cpr = d / 8;
+  const int64_t total = T * cpr;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t t = i / cpr;
+    const int c = (int)(i % cpr) * 8;
+    int id = ids[t];
+    id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+    *reinterpret_cast<u32x4*>(out + t * d + c) = *reinterpret_cast<const u32x4*>(W + (int64_t)id * d + c);
+  }
+}
+__global__ void embed_fwd_scalar(const int32_t* ids, const bf16* W, bf16* out, int64_t T, int d, int V) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= T * d) return;
+  int id = ids[i / d];
+  id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+  out[i] = W[(int64_t)id * d + i % d];
+}
+// dW[ids[t], :] += dh[t, :]   (fp32 accumulate; duplicates sum through atomics)
+__global__ __launch_bounds__(256) void embed_bwd_kernel(const int32_t* __restrict__ ids,
+                                                        const bf16* __restrict__ dh,
+                                                        float* __restrict__ dW, int64_t T, int d,
+                                                        int V) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < T * d; i += (int64_t)gridDim.x * 256) {
+    const int64_t t = i / d;
+    const int c = (int)(i % d);
+    int id = ids[t];
+    if (id < 0 || id >= V) continue;
+    atomicAdd(&dW[(int64_t)id * d + c], bf2f(dh[i]));
+  }
+}
+
+// ------------------------------------------------------------------ AdamW
+// p, m, v fp32 in place; g bf16 or fp32; optional bf16 working copy of the new p.
+// bc1 = 1 - b1^t, bc2 = 1 - b2^t (computed on the host in double).
+template <bool G_BF16>
+__global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ p, const void* __restrict__ gv,
+                                                    float* __restrict__ m, float* __restrict__ v,
+                                                    bf16* __restrict__ shadow, int64_t n, float lr,
+                                                    float b1, float b2, float eps, float wd,
+                                                    float bc1, float bc2, float gscale) {
+  const int64_t n4 = n / 4;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+    f32x4 pv = reinterpret_cast<const f32x4*>(p)[i];
+    f32x4 mv = reinterpret_cast<const f32x4*>(m)[i];
+    f32x4 vv = reinterpret_cast<const f32x4*>(v)[i];
+    float g[4];
+    if (G_BF16) {
+      Pack4 gp;
+      gp.u = reinterpret_cast<const u32x2*>(gv)[i];
+#pragma unroll
+      for (int e = 0; e < 4; e++) g[e] = bf2f(gp.e[e]);
+    } else {
+      f32x4 gf = reinterpret_cast<const f32x4*>(gv)[i];
+#pragma unroll
+      for (int e = 0; e < 4; e++) g[e] = gf[e];
+    }
+    Pack4 sh;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float ge = g[e] * gscale;
+      mv[e] = b1 * mv[e] + (1.f - b1) * ge;
+      vv[e] = b2 * vv[e] + (1.f - b2) * ge * ge;
+      const float mh = mv[e] / bc1;
+      const float vh = vv[e] / bc2;
+      pv[e] = pv[e] - lr * (mh / (sqrtf(vh) + eps) + wd * pv[e]);
+      sh.e[e] = f2bf(pv[e]);
+    }
+    reinterpret_cast<f32x4*>(p)[i] = pv;
+    reinterpret_cast<f32x4*>(m)[i] = mv;
+    reinterpret_cast<f32x4*>(v)[i] = vv;
+    if (shadow) reinterpret_cast<u32x2*>(shadow)[i] = sh.u;
+  }
+  // tail (n % 4) handled by the first threads of block 0
+  if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    const int64_t i = n4 * 4 + threadIdx.x;
+    const float ge = (G_BF16 ? bf2f(reinterpret_cast<const bf16*>(gv)[i]) : reinterpret_cast<const float*>(gv)[i]) * gscale;
+    const float mm = b1 * m[i] + (1.f - b1) * ge;
+    const float vv = b2 * v[i] + (1.f - b2) * ge * ge;
+    const float pp = p[i] - lr * ((mm / bc1) / (sqrtf(vv / bc2) + eps) + wd * p[i]);
+    m[i] = mm;
+    v[i] = vv;
+    p[i] = pp;
+    if (shadow) shadow[i] = f2bf(pp);
+  }
+}
+
+// sum of squares of a gradient leaf, accumulated (fp32 atomics) into *out
+template <bool G_BF16>
+__global__ __launch_bounds__(256) void sumsq_kernel(const void* __restrict__ gv, int64_t n,
+                                                    float* __restrict__ out) {
+  __shared__ float red[4];
+  float s = 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const float g = G_BF16 ? bf2f(reinterpret_cast<const bf16*>(gv)[i]) : reinterpret_cast<const float*>(gv)[i];
+    s += g * g;
+  }
+  s = block_sum<4>(s, red);
+  if (threadIdx.x == 0) atomicAdd(out, s);
+}
+
+__global__ void cast_f32_bf16_kernel(const float* __restrict__ in, bf16* __restrict__ out, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    out[i] = f2bf(in[i]);
+}
+__global__ void cast_bf16_f32_kernel(const bf16* __restrict__ in, float* __restrict__ out, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    out[i] = bf2f(in[i]);
+}
+__global__ void fill_u32_kernel(uint32_t* __restrict__ p, uint32_t val, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    p[i] = val;
+}
+// out = a + b (bf16), 8 per lane
+__global__ __launch_bounds__(256) void add_bf16_kernel(const bf16* __restrict__ a, const bf16* __restrict__ b,
+                                                       bf16* __restrict__ out, int64_t n8) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+    Pack8 x, y, o;
+    x.u = reinterpret_cast<const u32x4*>(a)[i];
+    y.u = reinterpret_cast<const u32x4*>(b)[i];
+#pragma unroll
+    for (int e = 0; e < 8; e++) o.e[e] = f2bf(bf2f(x.e[e]) + bf2f(y.e[e]));
+    reinterpret_cast<u32x4*>(out)[i] = o.u;
+  }
+}
+
+int grid_1d(int64_t items, int cap = 8192) {
+  int64_t g = (items + 255) / 256;
+  return (int)(g < 1 ? 1 : (g > cap ? cap : g));
+}
+
+}  // namespace
+
+extern "C" int32_t olmax_glu_fwd(hipStream_t stream, const void* gate, const void* up, void* out,
+                                 int64_t T, int32_t F, int64_t ldg, int64_t ldu, int64_t ldo,
+                                 int32_t act) {
+  if (T == 0) return OLMAX_OK;
+  OLMAX_CHECK(gate && up && out, OLMAX_ERR_ARG, "olmax_glu_fwd: null pointer");
+  OLMAX_CHECK(T >= 0 && F > 0 && ldg >= F && ldu >= F && ldo >= F, OLMAX_ERR_SHAPE, "olmax_glu_fwd: bad shape");
+  OLMAX_CHECK(act == 0 || act == 1, OLMAX_ERR_ARG, "olmax_glu_fwd: act must be 0 (silu) or 1 (gelu-tanh)");
+  const bf16 *g = (const bf16*)gate, *u = (const bf16*)up;
+  bf16* o = (bf16*)out;
+  const bool vec = F % 8 == 0 && ldg % 8 == 0 && ldu % 8 == 0 && ldo % 8 == 0 && aligned16(gate) && aligned16(up) && aligned16(out);
+  if (vec) {
+    const int grid = grid_1d(T * (F / 8));
+    if (act) hipLaunchKernelGGL(glu_fwd_kernel<true>, dim3(grid), dim3(256), 0, stream, g, u, o, T, F, ldg, ldu, ldo);
+    else hipLaunchKernelGGL(glu_fwd_kernel<false>, dim3(grid), dim3(256), 0, stream, g, u, o, T, F, ldg, ldu, ldo);
+  } else {
+    const unsigned grid = (unsigned)((T * F + 255) / 256);
+    if (act) hipLaunchKernelGGL(glu_fwd_scalar<true>, dim3(grid), dim3(256), 0, stream, g, u, o, T, F, ldg, ldu, ldo);
+    else hipLaunchKernelGGL(glu_fwd_scalar<false>, dim3(grid), dim3(256), 0, stream, g, u, o, T, F, ldg, ldu, ldo);
+  }
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+extern "C" int32_t olmax_glu_bwd(hipStream_t stream, const void* gate, const void* up,
+                                 const void* dh, void* dgate, void* dup, int64_t T, int32_t F,
+                                 int64_t ldg, int64_t ldu, int64_t lddh, int64_t lddg, int64_t lddu,
+                                 int32_t act) {
+  if (T == 0) return OLMAX_OK;
+  OLMAX_CHECK(gate && up && dh && dgate && dup, OLMAX_ERR_ARG, "olmax_glu_bwd: null pointer");
+  OLMAX_CHECK(T >= 0 && F > 0 && ldg >= F && ldu >= F && lddh >= F && lddg >= F && lddu >= F, OLMAX_ERR_SHAPE, "olmax_glu_bwd: bad shape");
+  OLMAX_CHECK(act == 0 || act == 1, OLMAX_ERR_ARG, "olmax_glu_bwd: act must be 0 (silu) or 1 (gelu-tanh)");
+  const bf16 *g = (const bf16*)gate, *u = (const bf16*)up, *d = (const bf16*)dh;
+  bf16 *og = (bf16*)dgate, *ou = (bf16*)dup;
+  const bool vec = F % 8 == 0 && ldg % 8 == 0 && ldu % 8 == 0 && lddh % 8 == 0 && lddg % 8 == 0 && lddu % 8 == 0 &&
+                   aligned16(gate) && aligned16(up) && aligned16(dh) && aligned16(dgate) && aligned16(dup);
+  if (vec) {
+    const int grid = grid_1d(T * (F / 8));
+    if (act) hipLaunchKernelGGL(glu_bwd_kernel<true>, dim3(grid), dim3(256), 0, stream, g, u, d, og, ou, T, F, ldg, ldu, lddh, lddg, lddu);
+    else hipLaunchKernelGGL(glu_bwd_kernel<false>, dim3(grid), dim3(256), 0, stream, g, u, d, og, ou, T, F, ldg, ldu, lddh, lddg, lddu);
+  } else {
+    const unsigned grid = (unsigned)((T * F + 255) / 256);
+    if (act) hipLaunchKernelGGL(glu_bwd_scalar<true>, dim3(grid), dim3(256), 0, stream, g, u, d, og, ou, T, F, ldg, ldu, lddh, lddg, lddu);
+    else hipLaunchKernelGGL(glu_bwd_scalar<false>, dim3(grid), dim3(256), 0, stream, g, u, d, og, ou, T, F, ldg, ldu, lddh, lddg, lddu);
+  }
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+extern "C" int32_t olmax_embed_fwd(hipStream_t stream, const int32_t* ids, const void* W, void* out,
+                                   int64_t T, int32_t d, int32_t V) {
+  if (T == 0) return OLMAX_OK;
+  OLMAX_CHECK(ids && W && out, OLMAX_ERR_ARG, "olmax_embed_fwd: null pointer");
+  OLMAX_CHECK(T >= 0 && d > 0 && V > 0, OLMAX_ERR_SHAPE, "olmax_embed_fwd: bad shape");
+  if (d % 8 == 0 && aligned16(W) && aligned16(out))
+    hipLaunchKernelGGL(embed_fwd_kernel, dim3(grid_1d(T * (d / 8))), dim3(256), 0, stream, ids, (const bf16*)W, (bf16*)out, T, d, V);
+  else
+    hipLaunchKernelGGL(embed_fwd_scalar, dim3((unsigned)((T * d + 255) / 256)), dim3(256), 0, stream, ids, (const bf16*)W, (bf16*)out, T, d, V);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+// dW (fp32 [V, d]) is ACCUMULATED into: the caller zeroes it (or seeds it, for tied heads).
+extern "C" int32_t olmax_embed_bwd(hipStream_t stream, const int32_t* ids, const void* dh, float* dW,
+                                   int64_t T, int32_t d, int32_t V) {
+  if (T == 0) return OLMAX_OK;
+  OLMAX_CHECK(ids && dh && dW, OLMAX_ERR_ARG, "olmax_embed_bwd: null pointer");
+  OLMAX_CHECK(T >= 0 && d > 0 && V > 0, OLMAX_ERR_SHAPE, "olmax_embed_bwd: bad shape");
+  hipLaunchKernelGGL(embed_bwd_kernel, dim3(grid_1d(T * d)), dim3(256), 0, stream, ids, (const bf16*)dh, dW, T, d, V);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+extern "C" int32_t olmax_adamw(hipStream_t stream, float* p, const void* g, float* m, float* v,
+                               void* shadow_bf16, int64_t n, int32_t grad_is_bf16, float lr, float b1,
+                               float b2, float eps, float wd, int64_t step, float grad_scale) {
+  if (n == 0) return OLMAX_OK;
+  OLMAX_CHECK(p && g && m && v, OLMAX_ERR_ARG, "olmax_adamw: null pointer");
+  OLMAX_CHECK(n >= 0 && step >= 1, OLMAX_ERR_ARG, "olmax_adamw: n must be >= 0 and step >= 1 (1-based)");
+  OLMAX_CHECK(aligned16(p) && aligned16(m) && aligned16(v) && (((uintptr_t)g) & (grad_is_bf16 ? 7 : 15)) == 0 &&
+                  (!shadow_bf16 || (((uintptr_t)shadow_bf16) & 7) == 0),
+              OLMAX_ERR_ALIGN, "olmax_adamw: buffers must be 16-byte aligned (bf16 buffers 8-byte)");
+  const float bc1 = (float)(1.0 - pow((double)b1, (double)step));
+  const float bc2 = (float)(1.0 - pow((double)b2, (double)step));
+  const int grid = grid_1d((n + 3) / 4, 16384);
+  if (grad_is_bf16)
+    hipLaunchKernelGGL(adamw_kernel<true>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale);
+  else
+    hipLaunchKernelGGL(adamw_kernel<false>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+// *out (fp32 scalar) += sum(g^2); the caller zeroes it.
+extern "C" int32_t olmax_sumsq(hipStream_t stream, const void* g, int64_t n, int32_t is_bf16, float* out) {
+  if (n == 0) return OLMAX_OK;
+  OLMAX_CHECK(g && out && n >= 0, OLMAX_ERR_ARG, "olmax_sumsq: bad argument");
+  const int grid = grid_1d(n, 2048);
+  if (is_bf16) hipLaunchKernelGGL(sumsq_kernel<true>, dim3(grid), dim3(256), 0, stream, g, n, out);
+  else hipLaunchKernelGGL(sumsq_kernel<false>, dim3(grid), dim3(256), 0, stream, g, n, out);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+extern "C" int32_t olmax_cast_f32_to_bf16(hipStream_t stream, const float* in, void* out, int64_t n) {
+  if (n == 0) return OLMAX_OK;
+  OLMAX_CHECK(in && out && n >= 0, OLMAX_ERR_ARG, "olmax_cast_f32_to_bf16: bad argument");
+  hipLaunchKernelGGL(cast_f32_bf16_kernel, dim3(grid_1d(n)), dim3(256), 0, stream, in, (bf16*)out, n);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+extern "C" int32_t olmax_cast_bf16_to_f32(hipStream_t stream, const void* in, float* out, int64_t n) {
+  if (n == 0) return OLMAX_OK;
+  OLMAX_CHECK(in && out && n >= 0, OLMAX_ERR_ARG, "olmax_cast_bf16_to_f32: bad argument");
+  hipLaunchKernelGGL(cast_bf16_f32_kernel, dim3(grid_1d(n)), dim3(256), 0, stream, (const bf16*)in, out, n);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+// Fill kernel (graph-capture safe replacement for memset); nbytes must be a multiple of 4.
+extern "C" int32_t olmax_fill_zero(hipStream_t stream, void* p, int64_t nbytes) {
+  OLMAX_CHECK(p && nbytes >= 0 && nbytes % 4 == 0 && (((uintptr_t)p) & 3) == 0, OLMAX_ERR_ARG, "olmax_fill_zero: need 4-byte aligned pointer and size");
+  if (nbytes == 0) return OLMAX_OK;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_1d(nbytes / 4)), dim3(256), 0, stream, (uint32_t*)p, 0u, nbytes / 4);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+extern "C" int32_t olmax_add_bf16(hipStream_t stream, const void* a, const void* b, void* out, int64_t n) {
+  if (n == 0) return OLMAX_OK;
+  OLMAX_CHECK(a && b && out && n >= 0 && n % 8 == 0 && aligned16(a) && aligned16(b) && aligned16(out), OLMAX_ERR_ARG, "olmax_add_bf16: need n % 8 == 0 and 16-byte alignment");
+  hipLaunchKernelGGL(add_bf16_kernel, dim3(grid_1d(n / 8)), dim3(256), 0, stream, (const bf16*)a, (const bf16*)b, (bf16*)out, n / 8);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}

@@ -1,0 +1,240 @@
+// Cross-entropy over the full vocabulary and the fused LM-head + CE forward/backward.
+//
+// Reference semantics: cross_entropy_loss, src/olmax/nn/functional.py:70-91 (reduction
+// "mean" over labels != ignore_index; an out-of-range label contributes zero loss and zero
+// gradient but still counts in the denominator), fed by LMHead.forward,
+// src/olmax/nn/lm_head.py:59-61 (logits = bf16 GEMM output widened to fp32).
+//
+// One 256-thread block owns one row of logits: pass 1 streams the row with 128-bit loads
+// keeping an online (max, sum-exp) per lane and reduces with wave shuffles; pass 2 re-reads
+// the row (L2-resident: a 100k-entry bf16 row is 200 KB) and overwrites it with
+// d logits = (softmax - onehot) * dloss / n_counted.  Optional final-logit soft-cap
+// z = c*tanh(x/c) is applied on the fly in both passes.
+#include "common.h"
+
+extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void* B, void* C,
+                                   const void* R, int32_t M, int32_t N, int32_t K, int64_t lda,
+                                   int64_t ldb, int64_t ldc, int64_t ldr, int32_t a_layout,
+                                   int32_t b_layout, int32_t out_f32);
+
+namespace {
+
+__global__ __launch_bounds__(256) void ce_count_kernel(const int32_t* __restrict__ labels, int64_t T,
+                                                       int32_t ignore_index, int32_t* __restrict__ n_out) {
+  __shared__ float red[4];
+  float c = 0.f;
+  for (int64_t i = threadIdx.x; i < T; i += 256) c += labels[i] != ignore_index ? 1.f : 0.f;
+  c = block_sum<4>(c, red);
+  if (threadIdx.x == 0) *n_out = (int32_t)(c + 0.5f);
+}
+
+template <typename T> struct Io;
+template <> struct Io<bf16> {
+  static constexpr int VEC = 8;
+  static __device__ __forceinline__ void load(const bf16* p, float* f) {
+    Pack8 t;
+    t.u = *reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+    for (int e = 0; e < 8; e++) f[e] = bf2f(t.e[e]);
+  }
+  static __device__ __forceinline__ void store(bf16* p, const float* f) {
+    Pack8 t;
+#pragma unroll
+    for (int e = 0; e < 8; e++) t.e[e] = f2bf(f[e]);
+    *reinterpret_cast<u32x4*>(p) = t.u;
+  }
+  static __device__ __forceinline__ float ld1(const bf16* p) { return bf2f(*p); }
+  static __device__ __forceinline__ void st1(bf16* p, float f) { *p = f2bf(f); }
+};
+template <> struct Io<float> {
+  static constexpr int VEC = 4;
+  static __device__ __forceinline__ void load(const float* p, float* f) {
+    f32x4 t = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+    for (int e = 0; e < 4; e++) f[e] = t[e];
+  }
+  static __device__ __forceinline__ void store(float* p, const float* f) {
+    f32x4 t;
+#pragma unroll
+    for (int e = 0; e < 4; e++) t[e] = f[e];
+    *reinterpret_cast<f32x4*>(p) = t;
+  }
+  static __device__ __forceinline__ float ld1(const float* p) { return *p; }
+  static __device__ __forceinline__ void st1(float* p, float f) { *p = f; }
+};
+
+template <typename T, bool CAP>
+__global__ __launch_bounds__(256) void ce_row_kernel(
+    const T* __restrict__ logits, T* __restrict__ dlogits, const int32_t* __restrict__ labels,
+    float* __restrict__ row_loss, float* __restrict__ lse_out, const int32_t* __restrict__ n_counted,
+    int64_t rows, int V, int64_t ld, int64_t ldd, int32_t ignore_index, float cap, float dloss,
+    int vec_ok) {
+  constexpr int VEC = Io<T>::VEC;
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const T* zr = logits + row * ld;
+  const int label = labels[row];
+  const float inv_cap = CAP ? 1.f / cap : 0.f;
+  // ---- pass 1: online max / sum-exp ----
+  float mx = -INFINITY, sm = 0.f;
+  const int nvec = vec_ok ? V / VEC : 0;
+  for (int i = threadIdx.x; i < nvec; i += 256) {
+    float f[VEC];
+    Io<T>::load(zr + i * VEC, f);
+    float cm = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      if (CAP) f[e] = cap * tanhf(f[e] * inv_cap);
+      cm = fmaxf(cm, f[e]);
+    }
+    if (cm > mx) {
+      sm *= __expf(mx - cm);
+      mx = cm;
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; e++) sm += __expf(f[e] - mx);
+  }
+  for (int i = nvec * VEC + threadIdx.x; i < V; i += 256) {
+    float f = Io<T>::ld1(zr + i);
+    if (CAP) f = cap * tanhf(f * inv_cap);
+    if (f > mx) {
+      sm *= __expf(mx - f);
+      mx = f;
+    }
+    sm += __expf(f - mx);
+  }
+  const float gmx = block_max<4>(mx, red);
+  sm = (mx == -INFINITY) ? 0.f : sm * __expf(mx - gmx);
+  const float gsm = block_sum<4>(sm, red);
+  const float lse = gmx + __logf(gsm);
+  const bool counted = label != ignore_index;
+  const bool inrange = label >= 0 && label < V;
+  if (threadIdx.x == 0) {
+    float zl = 0.f;
+    if (counted && inrange) {
+      zl = Io<T>::ld1(zr + label);
+      if (CAP) zl = cap * tanhf(zl * inv_cap);
+    }
+    row_loss[row] = (counted && inrange) ? (lse - zl) : 0.f;
+    if (lse_out) lse_out[row] = counted ? lse : 0.f;
+  }
+  if (!dlogits) return;
+  // ---- pass 2: gradient, in place allowed ----
+  T* dr = dlogits + row * ldd;
+  const float scale = (counted && inrange) ? dloss / (float)(*n_counted) : 0.f;
+  for (int i = threadIdx.x; i < nvec; i += 256) {
+    float f[VEC];
+    Io<T>::load(zr + i * VEC, f);
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      float z = f[e], chain = 1.f;
+      if (CAP) {
+        const float t = tanhf(z * inv_cap);
+        z = cap * t;
+        chain = 1.f - t * t;
+      }
+      float p = __expf(z - lse);
+      if (i * VEC + e == label) p -= 1.f;
+      f[e] = p * scale * chain;
+    }
+    Io<T>::store(dr + i * VEC, f);
+  }
+  for (int i = nvec * VEC + threadIdx.x; i < V; i += 256) {
+    float z = Io<T>::ld1(zr + i), chain = 1.f;
+    if (CAP) {
+      const float t = tanhf(z * inv_cap);
+      z = cap * t;
+      chain = 1.f - t * t;
+    }
+    float p = __expf(z - lse);
+    if (i == label) p -= 1.f;
+    Io<T>::st1(dr + i, p * scale * chain);
+  }
+}
+
+// loss = sum(row_loss) / n_counted   (single block; deterministic order)
+__global__ __launch_bounds__(256) void ce_finalize_kernel(const float* __restrict__ row_loss, int64_t T,
+                                                          const int32_t* __restrict__ n_counted,
+                                                          float* __restrict__ loss) {
+  __shared__ float red[4];
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < T; i += 256) s += row_loss[i];
+  s = block_sum<4>(s, red);
+  if (threadIdx.x == 0) *loss = s / (float)(*n_counted);
+}
+
+}  // namespace
+
+// Workspace: T floats (row losses) + 16 bytes (counted-row count), 16-byte aligned.
+extern "C" int64_t olmax_cross_entropy_workspace_bytes(int64_t T) { return ((T * 4 + 15) / 16) * 16 + 16; }
+
+// logits [T, V] (bf16 when logits_f32 == 0, else fp32) -> *loss (fp32 scalar, device);
+// dlogits (same dtype, may alias logits, may be NULL) <- d loss / d logits * dloss;
+// lse_out (optional, [T]) <- log-normaliser * (label != ignore_index)  (the reference's
+// fused_cross_entropy_loss second output, src/olmax/nn/functional.py:94-121).
+extern "C" int32_t olmax_cross_entropy(hipStream_t stream, const void* logits, void* dlogits,
+                                       const int32_t* labels, float* loss, float* lse_out,
+                                       void* workspace, int64_t workspace_bytes, int64_t T, int32_t V,
+                                       int64_t ld, int64_t ldd, int32_t logits_f32,
+                                       int32_t ignore_index, float softcap, float dloss) {
+  OLMAX_CHECK(logits && labels && loss && workspace, OLMAX_ERR_ARG, "olmax_cross_entropy: null pointer");
+  OLMAX_CHECK(T > 0 && V > 0 && ld >= V && (!dlogits || ldd >= V), OLMAX_ERR_SHAPE, "olmax_cross_entropy: bad shape T=%ld V=%d", (long)T, V);
+  OLMAX_CHECK(workspace_bytes >= olmax_cross_entropy_workspace_bytes(T) && aligned16(workspace), OLMAX_ERR_WORKSPACE, "olmax_cross_entropy: workspace too small or misaligned");
+  float* row_loss = (float*)workspace;
+  int32_t* n_counted = (int32_t*)((char*)workspace + ((T * 4 + 15) / 16) * 16);
+  hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(256), 0, stream, labels, T, ignore_index, n_counted);
+  const int vecw = logits_f32 ? 4 : 8;
+  const int vec_ok = aligned16(logits) && (!dlogits || aligned16(dlogits)) && ld % vecw == 0 && (!dlogits || ldd % vecw == 0);
+  const bool cap = softcap > 0.f;
+  dim3 grid((unsigned)T);
+#define CE_GO(TY, CAPV)                                                                          \
+  hipLaunchKernelGGL((ce_row_kernel<TY, CAPV>), grid, dim3(256), 0, stream, (const TY*)logits,   \
+                     (TY*)dlogits, labels, row_loss, lse_out, n_counted, T, V, ld, ldd,          \
+                     ignore_index, softcap, dloss, vec_ok)
+  if (logits_f32) {
+    if (cap) CE_GO(float, true); else CE_GO(float, false);
+  } else {
+    if (cap) CE_GO(bf16, true); else CE_GO(bf16, false);
+  }
+#undef CE_GO
+  hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(256), 0, stream, row_loss, T, n_counted, loss);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+// Workspace for the fused LM head: bf16 logits [T, V] + the CE workspace.
+extern "C" int64_t olmax_lmhead_ce_workspace_bytes(int64_t T, int32_t V) {
+  return ((T * (int64_t)V * 2 + 255) / 256) * 256 + olmax_cross_entropy_workspace_bytes(T);
+}
+
+// Fused LM head + cross entropy, forward and backward in one call:
+//   logits = h W^T (bf16) ; loss = CE(softcap(logits), labels) ;
+//   dlogits overwrites logits in the workspace ; dh = dlogits W ; dW = dlogits^T h.
+// h [T, d] bf16, W [V, d] bf16, labels [T] int32.  dh [T, d] bf16 and dW [V, d] (bf16, or
+// fp32 when dw_f32 != 0) may be NULL to skip that product (forward-only when both are NULL).
+extern "C" int32_t olmax_lmhead_ce(hipStream_t stream, const void* h, const void* W,
+                                   const int32_t* labels, float* loss, void* dh, void* dW,
+                                   void* workspace, int64_t workspace_bytes, int64_t T, int32_t d,
+                                   int32_t V, int32_t ignore_index, float softcap, int32_t dw_f32) {
+  OLMAX_CHECK(h && W && labels && loss && workspace, OLMAX_ERR_ARG, "olmax_lmhead_ce: null pointer");
+  OLMAX_CHECK(T > 0 && d > 0 && V > 0 && T < (1LL << 31), OLMAX_ERR_SHAPE, "olmax_lmhead_ce: bad shape");
+  OLMAX_CHECK(workspace_bytes >= olmax_lmhead_ce_workspace_bytes(T, V) && (((uintptr_t)workspace) & 255) == 0, OLMAX_ERR_WORKSPACE,
+              "olmax_lmhead_ce: workspace needs %ld bytes, 256-byte aligned", (long)olmax_lmhead_ce_workspace_bytes(T, V));
+  void* logits = workspace;
+  void* ce_ws = (char*)workspace + ((T * (int64_t)V * 2 + 255) / 256) * 256;
+  int rc = olmax_gemm_bf16(stream, h, W, logits, nullptr, (int)T, V, d, d, d, V, 0, 0, 0, 0);
+  if (rc) return rc;
+  const bool need_grad = dh || dW;
+  rc = olmax_cross_entropy(stream, logits, need_grad ? logits : nullptr, labels, loss, nullptr, ce_ws,
+                           olmax_cross_entropy_workspace_bytes(T), T, V, V, V, 0, ignore_index, softcap, 1.f);
+  if (rc) return rc;
+  if (dh) {
+    rc = olmax_gemm_bf16(stream, logits, W, dh, nullptr, (int)T, d, V, V, d, d, 0, 0, 1, 0);
+    if (rc) return rc;
+  }
+  if (dW) {
+    rc = olmax_gemm_bf16(stream, logits, h, dW, nullptr, V, d, (int)T, V, d, d, 0, 1, 1, dw_f32);
+    if (rc) return rc;
+  }
+  return OLMAX_OK;
+}

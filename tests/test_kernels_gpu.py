@@ -1,0 +1,312 @@
+"""GPU parity tests: every HIP entry point, called through the C ABI, against the CPU oracle
+on the same seeded inputs.  Tolerances follow the stated gates: activations within 1e-2
+relative (bf16), gradient cosine similarity >= 0.999; integer/index work bit-exact."""
+import math
+import sys
+
+import pytest
+import torch
+
+from oracle import ref
+
+pytestmark = pytest.mark.gpu
+
+BF = torch.bfloat16
+rt = ref.bf16_round
+
+
+def _ops():
+    from olmax_amd import ops
+    return ops
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+def relerr(got: torch.Tensor, want: torch.Tensor) -> float:
+    got, want = got.double().cpu(), want.double().cpu()
+    return ((got - want).norm() / (want.norm() + 1e-30)).item()
+
+
+def maxrel(got, want) -> float:
+    got, want = got.double().cpu(), want.double().cpu()
+    return ((got - want).abs().max() / (want.abs().max() + 1e-30)).item()
+
+
+def cosine(a, b) -> float:
+    a, b = a.double().cpu().flatten(), b.double().cpu().flatten()
+    return (a @ b / (a.norm() * b.norm() + 1e-30)).item()
+
+
+def bfr(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(BF)
+
+
+def check_close(got, want, name, tol=1e-2, cos=0.9999):
+    e, c = relerr(got, want), cosine(got, want)
+    assert e < tol and c > cos, f"{name}: relerr {e:.3e} cosine {c:.6f}"
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 512, 128), (384, 128, 192), (1024, 2048, 512), (50, 36, 20), (129, 257, 65)])
+@pytest.mark.parametrize("al,bl", [(0, 0), (0, 1), (1, 1), (1, 0)])
+def test_gemm_layouts(M, N, K, al, bl):
+    ops = _ops()
+    say(f"gemm M{M} N{N} K{K} a{al} b{bl}")
+    a = bfr(*((M, K) if al == 0 else (K, M)), seed=1)
+    b = bfr(*((N, K) if bl == 0 else (K, N)), seed=2)
+    r = bfr(M, N, seed=3)
+    af = a.double() if al == 0 else a.double().t()
+    bf_ = b.double() if bl == 0 else b.double().t()
+    want = af @ bf_.t()
+    got = ops.gemm(a.cuda(), b.cuda(), a_layout=al, b_layout=bl)
+    assert maxrel(got, want) < 6e-3
+    got = ops.gemm(a.cuda(), b.cuda(), a_layout=al, b_layout=bl, residual=r.cuda(), out_f32=True)
+    assert maxrel(got, want + r.double()) < 1e-5
+
+
+def test_gemm_brute_force_tiny_and_strided():
+    ops = _ops()
+    say("gemm tiny brute force + strided views")
+    a = bfr(3, 5, seed=4); b = bfr(4, 5, seed=5)
+    got = ops.gemm(a.cuda(), b.cuda(), out_f32=True).cpu()
+    for i in range(3):
+        for j in range(4):
+            assert abs(got[i, j].item() - sum(float(a[i, k]) * float(b[j, k]) for k in range(5))) < 1e-5
+    # row-strided operands (column slices of wider buffers), MFMA path
+    big_a = bfr(256, 512, seed=6).cuda(); big_b = bfr(256, 384, seed=7).cuda()
+    av, bv = big_a[:, 128:384], big_b[:, 64:320]
+    got = ops.gemm(av, bv)
+    assert maxrel(got, av.double().cpu() @ bv.double().cpu().t()) < 6e-3
+
+
+def test_gemm_rejects_bad_arguments():
+    ops = _ops()
+    from olmax_amd._lib import OlmaxHipError
+    with pytest.raises(AssertionError):
+        ops.gemm(bfr(4, 5).cuda(), bfr(4, 6).cuda())
+    with pytest.raises(OlmaxHipError):
+        ops.gemm(bfr(4, 5), bfr(4, 5))  # CPU tensors: no fallback
+
+
+@pytest.mark.parametrize("rows,d", [(64, 4096), (37, 256), (130, 128), (16, 5376), (9, 4608), (5, 100), (3, 16)])
+def test_rmsnorm(rows, d):
+    ops = _ops()
+    say(f"rmsnorm rows{rows} d{d}")
+    x = bfr(rows, d, seed=1); w = (1 + 0.1 * torch.randn(d, generator=torch.Generator().manual_seed(2))).to(BF)
+    dy = bfr(rows, d, seed=3); dres = bfr(rows, d, seed=4)
+    y = ops.rms_norm_fwd(x.cuda(), w.cuda(), 1e-6)
+    want = ref.rms_norm_fwd(x.double(), w.double(), 1e-6)
+    assert maxrel(y, want) < 1e-2
+    dx, dw = ops.rms_norm_bwd(x.cuda(), w.cuda(), dy.cuda(), 1e-6)
+    wdx, wdw = ref.rms_norm_bwd(x.double(), w.double(), dy.double(), 1e-6)
+    check_close(dx, wdx, "dx"); check_close(dw, wdw, "dw")
+    dx2, _ = ops.rms_norm_bwd(x.cuda(), w.cuda(), dy.cuda(), 1e-6, dres=dres.cuda())
+    check_close(dx2, wdx + dres.double(), "dx+dres")
+    # no weight
+    y0 = ops.rms_norm_fwd(x.cuda(), None, 1e-6)
+    assert maxrel(y0, ref.rms_norm_fwd(x.double(), None, 1e-6)) < 1e-2
+
+
+def test_rmsnorm_empty_and_strided():
+    ops = _ops()
+    say("rmsnorm empty + strided")
+    x = torch.empty(0, 128, dtype=BF).cuda()
+    assert ops.rms_norm_fwd(x, None, 1e-6).shape == (0, 128)
+    big = bfr(32, 1024, seed=5).cuda()
+    v = big[:, 256:768]
+    y = ops.rms_norm_fwd(v, None, 1e-5)
+    assert maxrel(y, ref.rms_norm_fwd(v.double().cpu(), None, 1e-5)) < 1e-2
+
+
+@pytest.mark.parametrize("D,heads,norm", [(128, 4, False), (128, 3, True), (64, 4, False), (16, 2, True)])
+def test_qk_rope(D, heads, norm):
+    ops = _ops()
+    say(f"qk_rope D{D} heads{heads} norm{norm}")
+    B, S = 2, 24
+    x = bfr(B * S, heads * D, seed=1); dy = bfr(B * S, heads * D, seed=2)
+    w = (1 + 0.1 * torch.randn(D, generator=torch.Generator().manual_seed(3))).to(BF) if norm else None
+    cos, sin = ops.rope_tables(S, D, 500000.0, "cuda")
+    rc, rs = ref.rope_tables(S, D, 500000.0)
+    assert torch.equal(cos.cpu(), rc) and torch.equal(sin.cpu(), rs)  # positions/tables bit-exact
+    y = ops.qk_rope_fwd(x.cuda(), cos, sin, heads=heads, head_dim=D, seq_len=S, w=None if w is None else w.cuda())
+    x4 = x.double().reshape(B, S, heads, D)
+    xn = rt(ref.rms_norm_fwd(x4, w.double(), 1e-6)) if norm else x4
+    want = ref.rope_fwd(xn, rc.double(), rs.double()).reshape(B * S, heads * D)
+    assert maxrel(y, want) < 1e-2
+    dx, dw = ops.qk_rope_bwd(dy.cuda(), cos, sin, heads=heads, head_dim=D, seq_len=S,
+                             x=x.cuda() if norm else None, w=None if w is None else w.cuda())
+    g = ref.rope_bwd(dy.double().reshape(B, S, heads, D), rc.double(), rs.double())
+    if norm:
+        g, wdw = ref.rms_norm_bwd(x4, w.double(), rt(g), 1e-6)
+        check_close(dw, wdw, "dw")
+    check_close(dx, g.reshape(B * S, heads * D), "dx")
+
+
+def test_qk_rope_inplace_on_strided_qkv():
+    ops = _ops()
+    say("qk_rope in place on a fused qkv buffer")
+    B, S, H, D = 1, 16, 2, 128
+    qkv = bfr(B * S, 3 * H * D, seed=7).cuda()
+    orig = qkv.clone()
+    cos, sin = ops.rope_tables(S, D, 1e4, "cuda")
+    qv = qkv[:, : H * D]
+    ops.qk_rope_fwd(qv, cos, sin, heads=H, head_dim=D, seq_len=S, out=qv)
+    rc, rs = ref.rope_tables(S, D, 1e4)
+    want = ref.rope_fwd(orig[:, : H * D].double().cpu().reshape(B, S, H, D), rc.double(), rs.double()).reshape(B * S, H * D)
+    assert maxrel(qkv[:, : H * D], want) < 1e-2
+    assert torch.equal(qkv[:, H * D:], orig[:, H * D:])  # k, v untouched
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("T,F", [(64, 1024), (7, 24), (5, 11)])
+def test_glu(act, T, F):
+    ops = _ops()
+    say(f"glu {act} T{T} F{F}")
+    gu = bfr(T, 2 * F, seed=1, scale=2.0); dh = bfr(T, F, seed=2)
+    g, u = gu[:, :F], gu[:, F:]
+    gc = gu.cuda()
+    out = ops.glu_fwd(gc[:, :F], gc[:, F:], act)
+    assert maxrel(out, ref.glu_fwd(g.double(), u.double(), act, rt)) < 1e-2
+    dg, du = ops.glu_bwd(gc[:, :F], gc[:, F:], dh.cuda(), act)
+    wg, wu = ref.glu_bwd(g.double(), u.double(), dh.double(), act)
+    check_close(dg, wg, "dgate"); check_close(du, wu, "dup")
+
+
+ATTN_CASES = [
+    # B, S, H, KH, D, window, softcap
+    (2, 256, 4, 4, 128, None, 0.0),
+    (1, 384, 4, 2, 128, None, 0.0),
+    (1, 320, 4, 2, 128, 100, 0.0),
+    (1, 256, 2, 1, 128, 64, 30.0),
+    (1, 200, 2, 2, 128, None, 0.0),     # ragged: not a multiple of the tile
+    (1, 130, 2, 1, 128, 7, 0.0),
+    (2, 48, 4, 4, 64, None, 0.0),       # generic head_dim path
+    (1, 40, 4, 2, 16, 9, 5.0),
+]
+
+
+@pytest.mark.parametrize("B,S,H,KH,D,window,softcap", ATTN_CASES)
+def test_attention_fwd_bwd(B, S, H, KH, D, window, softcap):
+    ops = _ops()
+    say(f"attn B{B} S{S} H{H} KH{KH} D{D} w{window} cap{softcap}")
+    q = bfr(B * S, H * D, seed=1); k = bfr(B * S, KH * D, seed=2); v = bfr(B * S, KH * D, seed=3)
+    do = bfr(B * S, H * D, seed=4)
+    o, lse = ops.attn_fwd(q.cuda(), k.cuda(), v.cuda(), B=B, S=S, H=H, KH=KH, D=D, window=window, softcap=softcap)
+    q4, k4, v4 = q.double().reshape(B, S, H, D), k.double().reshape(B, S, KH, D), v.double().reshape(B, S, KH, D)
+    wo, wlse = ref.attention_fwd(q4, k4, v4, window=window, softcap=softcap)
+    assert maxrel(o, wo.reshape(B * S, H * D)) < 1e-2, "o"
+    assert (lse.cpu().double() - wlse).abs().max() < 2e-3, "lse"
+    # first query attends to key 0 only
+    assert maxrel(o.reshape(B, S, H, D)[:, 0], v4.repeat_interleave(H // KH, 2)[:, 0]) < 1e-2
+    dq, dk, dv = ops.attn_bwd(q.cuda(), k.cuda(), v.cuda(), o, lse, do.cuda(), B=B, S=S, H=H, KH=KH, D=D,
+                              window=window, softcap=softcap)
+    wdq, wdk, wdv = ref.attention_bwd(q4, k4, v4, wo, wlse, do.double().reshape(B, S, H, D), window=window, softcap=softcap)
+    check_close(dq, wdq.reshape(B * S, H * D), "dq", tol=2e-2, cos=0.999)
+    check_close(dk, wdk.reshape(B * S, KH * D), "dk", tol=2e-2, cos=0.999)
+    check_close(dv, wdv.reshape(B * S, KH * D), "dv", tol=2e-2, cos=0.999)
+
+
+def test_attention_on_strided_qkv_views():
+    ops = _ops()
+    say("attn on fused-qkv column views")
+    B, S, H, KH, D = 1, 256, 4, 2, 128
+    qkv = bfr(B * S, (H + 2 * KH) * D, seed=9).cuda()
+    q, k, v = qkv[:, : H * D], qkv[:, H * D:(H + KH) * D], qkv[:, (H + KH) * D:]
+    o, lse = ops.attn_fwd(q, k, v, B=B, S=S, H=H, KH=KH, D=D)
+    o2, lse2 = ops.attn_fwd(q.contiguous(), k.contiguous(), v.contiguous(), B=B, S=S, H=H, KH=KH, D=D)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
+
+
+@pytest.mark.parametrize("T,V,f32", [(33, 4096, False), (17, 1000, True), (8, 50, False), (5, 100352, False)])
+@pytest.mark.parametrize("cap", [0.0, 30.0])
+def test_cross_entropy(T, V, f32, cap):
+    ops = _ops()
+    say(f"ce T{T} V{V} f32{f32} cap{cap}")
+    g = torch.Generator().manual_seed(1)
+    logits = (torch.randn(T, V, generator=g) * 3)
+    logits = logits if f32 else logits.to(BF)
+    labels = torch.randint(0, V, (T,), generator=g, dtype=torch.int32)
+    labels[1] = -100
+    labels[2] = V  # out of range: zero loss, zero grad, counted
+    loss, d, lse = ops.cross_entropy(logits.cuda(), labels.cuda(), softcap=cap)
+    wl, wlse, n = ref.cross_entropy_fwd(logits.double(), labels.long(), softcap=cap)
+    assert abs(loss.item() - wl.item()) < 2e-3 * max(1.0, abs(wl.item()))
+    wd = ref.cross_entropy_bwd(logits.double(), labels.long(), softcap=cap)
+    check_close(d, wd, "dlogits", tol=1e-2 if not f32 else 1e-4)
+    assert d[1].abs().max().item() == 0 and d[2].abs().max().item() == 0
+    mask = (labels != -100).double()
+    assert ((lse.cpu().double() - wlse * mask).abs().max()) < 2e-3
+
+
+def test_cross_entropy_reference_invariants():
+    """src/test/nn/functional_test.py:10-18: an appended ignore_index row leaves the mean unchanged."""
+    ops = _ops()
+    say("ce invariants")
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(6, 64, generator=g)
+    labels = torch.randint(0, 64, (6,), generator=g, dtype=torch.int32)
+    l1, _, _ = ops.cross_entropy(logits.cuda(), labels.cuda(), want_grad=False)
+    l2, _, lse = ops.cross_entropy(torch.cat([logits, torch.randn(1, 64, generator=g)]).cuda(),
+                                   torch.cat([labels, torch.tensor([-100], dtype=torch.int32)]).cuda(), want_grad=False)
+    assert abs(l1.item() - l2.item()) < 1e-6
+    lu, _, _ = ops.cross_entropy(torch.zeros(4, 64).cuda(), torch.tensor([0, 1, 2, 3], dtype=torch.int32).cuda(), want_grad=False)
+    assert abs(lu.item() - math.log(64)) < 1e-5
+
+
+@pytest.mark.parametrize("T,d,V,cap", [(256, 128, 1024, 0.0), (128, 256, 512, 30.0), (40, 24, 100, 0.0)])
+def test_lmhead_ce(T, d, V, cap):
+    ops = _ops()
+    say(f"lmhead_ce T{T} d{d} V{V} cap{cap}")
+    h = bfr(T, d, seed=1); W = bfr(V, d, seed=2, scale=0.1)
+    labels = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(3), dtype=torch.int32)
+    labels[0] = -100
+    loss, dh, dW = ops.lmhead_ce(h.cuda(), W.cuda(), labels.cuda(), softcap=cap)
+    wl, wdh, wdw = ref.lm_head_ce(h.double(), W.double(), labels.long(), softcap=cap, rt=rt)
+    assert abs(loss.item() - wl.item()) < 1e-2 * abs(wl.item())
+    check_close(dh, wdh, "dh", tol=2e-2, cos=0.999); check_close(dW, wdw, "dW", tol=2e-2, cos=0.999)
+
+
+def test_embedding():
+    ops = _ops()
+    say("embedding gather / scatter-add")
+    V, d = 50, 64
+    W = bfr(V, d, seed=1)
+    ids = torch.tensor([3, 7, 3, 49, 0, 3], dtype=torch.int32)
+    out = ops.embed_fwd(ids.cuda(), W.cuda())
+    assert torch.equal(out.cpu(), W[ids.long()])  # index work is bit-exact
+    dh = bfr(6, d, seed=2)
+    dW = ops.embed_bwd(ids.cuda(), dh.cuda(), V)
+    want = ref.embed_bwd(ids, dh.double(), V)
+    assert (dW.cpu().double() - want).abs().max() < 1e-5
+    # odd width goes through the scalar path
+    W2 = bfr(V, 13, seed=3)
+    assert torch.equal(ops.embed_fwd(ids.cuda(), W2.cuda()).cpu(), W2[ids.long()])
+
+
+@pytest.mark.parametrize("n,gbf", [(4096, True), (1003, False), (7, True)])
+def test_adamw(n, gbf):
+    ops = _ops()
+    say(f"adamw n{n} gbf16{gbf}")
+    gen = torch.Generator().manual_seed(1)
+    p = torch.randn(n, generator=gen); m = torch.zeros(n); v = torch.zeros(n)
+    pc, mc, vc = p.cuda(), m.cuda(), v.cuda()
+    sh = torch.empty(n, dtype=BF).cuda()
+    pd, md, vd = p.double(), m.double(), v.double()
+    for step in range(1, 4):
+        g = torch.randn(n, generator=gen) * 0.1
+        g = g.to(BF) if gbf else g
+        ops.adamw_(pc, g.cuda(), mc, vc, step=step, lr=3e-3, b1=0.9, b2=0.95, eps=1e-8, wd=0.1, shadow=sh)
+        pd, md, vd = ref.adamw_step(pd, g.double(), md, vd, step=step, lr=3e-3, b1=0.9, b2=0.95, eps=1e-8, wd=0.1)
+    assert (pc.cpu().double() - pd).abs().max() < 1e-5
+    assert (mc.cpu().double() - md).abs().max() < 1e-6 and (vc.cpu().double() - vd).abs().max() < 1e-7
+    assert torch.equal(sh.cpu(), pc.cpu().to(BF))
+    # g = 0 -> pure decoupled decay; wd = 0 and |g| >> eps at step 1 -> -lr * sign(g)
+    p0 = torch.full((8,), 2.0).cuda(); z = torch.zeros(8).cuda()
+    ops.adamw_(p0, torch.zeros(8).cuda(), z.clone(), z.clone(), step=1, lr=0.1, wd=0.5)
+    assert (p0.cpu() - 2.0 * 0.95).abs().max() < 1e-6
+    p1 = torch.zeros(8).cuda()
+    ops.adamw_(p1, torch.tensor([1., -2., 3., -4., 5., -6., 7., -8.]).cuda(), z.clone(), z.clone(), step=1, lr=0.1, wd=0.0)
+    assert (p1.cpu() - torch.tensor([-0.1, 0.1] * 4)).abs().max() < 1e-6
