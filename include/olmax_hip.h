@@ -1,0 +1,250 @@
+/*
+ * libolmax_hip — C ABI of the MI355X (gfx950) transformer training hot path.
+ *
+ * The reference (epwalsh/OLMax) is pure JAX: it has no FFI boundary of its own, its kernels
+ * come from XLA / cuBLASLt / cuDNN behind jax.jit.  Each entry point below replaces one of
+ * those dispatches and cites the reference function whose arithmetic it implements; these
+ * are the symbols a jax.ffi custom-call adapter (or any other host) binds.
+ *
+ * Conventions
+ *  - All pointers are device pointers unless stated; the caller owns every buffer.
+ *  - Work is only ENQUEUED on `stream`; no call synchronises or touches another stream.
+ *  - Matrices are row-major with an explicit row stride in ELEMENTS ("ld*"); the last
+ *    dimension is contiguous.  bf16 storage, fp32 accumulation and statistics.
+ *  - Return 0 on success; negative on an argument error detected on the host before any
+ *    launch (olmax_last_error_string() gives the thread-local message).  Nothing throws.
+ *  - Calls hold no mutable global state; except where noted they never allocate.
+ */
+#ifndef OLMAX_HIP_H
+#define OLMAX_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* olmax_stream_t; /* == hipStream_t */
+
+#define OLMAX_OK 0
+#define OLMAX_ERR_ARG (-1)
+#define OLMAX_ERR_SHAPE (-2)
+#define OLMAX_ERR_ALIGN (-3)
+#define OLMAX_ERR_LAUNCH (-4)
+#define OLMAX_ERR_WORKSPACE (-5)
+
+const char* olmax_last_error_string(void);
+int32_t olmax_abi_version(void);
+
+/* ---- Linear: olmax.nn.functional.linear, src/olmax/nn/functional.py:14-27 (y = x W^T) and
+ * the two products JAX autodiff derives from it (dx = dy W, dW = dy^T x).
+ * C[M,N] = A B^T (+ R).  a_layout/b_layout 0: operand stored with the reduction dimension
+ * contiguous (A [M,K], B [N,K]); 1: stored transposed (A [K,M], B [K,N]).
+ * R (optional bf16 [M,N]) is added in fp32 before the single rounding of C (residual add of
+ * src/olmax/nn/transformer/layer.py:86,90).  out_f32 != 0 writes C as fp32. */
+int32_t olmax_gemm_bf16(olmax_stream_t stream, const void* A, const void* B, void* C, const void* R,
+                        int32_t M, int32_t N, int32_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                        int64_t ldr, int32_t a_layout, int32_t b_layout, int32_t out_f32);
+/* Test/tuning hook: force the MFMA tile variant (0 = automatic). */
+void olmax_gemm_set_tile(int tile);
+
+/* ---- RMSNorm: rms_norm, src/olmax/nn/functional.py:51-67; RMSNorm.forward,
+ * src/olmax/nn/normalization.py:85-87.  w may be NULL (no scale). */
+int32_t olmax_rmsnorm_fwd(olmax_stream_t stream, const void* x, const void* w, void* y, int64_t rows,
+                          int32_t d, int64_t ldx, int64_t ldy, float eps);
+/* y = bf16(rms_norm(x, w)) + res : post-norm residual of ReorderedNormTransformerLayer /
+ * GemmaTransformerLayer, src/olmax/nn/transformer/layer.py:108,112,175,181. */
+int32_t olmax_rmsnorm_fwd_res(olmax_stream_t stream, const void* x, const void* w, const void* res,
+                              void* y, int64_t rows, int32_t d, int64_t ldx, int64_t ldres,
+                              int64_t ldy, float eps);
+/* Transpose of rms_norm.  dx = d(norm)/dx^T dy (+ dres); dw (fp32 [d], optional) is
+ * ACCUMULATED into with atomics: zero it first. */
+int32_t olmax_rmsnorm_bwd(olmax_stream_t stream, const void* x, const void* w, const void* dy,
+                          const void* dres, void* dx, float* dw, int64_t rows, int32_t d, int64_t ldx,
+                          int64_t lddy, int64_t lddres, int64_t lddx, float eps);
+
+/* ---- RoPE (+ head-wise QK-norm): RotaryPositionalEmbedding._apply_rope,
+ * src/olmax/nn/rope.py:99-115 (rotate_half, fp32), applied to q and k at
+ * src/olmax/nn/attention.py:298-300 after the optional head-wise norm of :293-296.
+ * x/y: [tokens, heads*head_dim] views (in place allowed); position = token % seq_len;
+ * cos/sin: fp32 [seq_len, head_dim/2] (precompute_freqs_cis, rope.py:118-145).
+ * w != NULL: y = rope(bf16(rms_norm_per_head(x, w))). */
+int32_t olmax_qk_rope_fwd(olmax_stream_t stream, const void* x, void* y, const void* w,
+                          const float* cos_t, const float* sin_t, int64_t tokens, int32_t heads,
+                          int32_t head_dim, int32_t seq_len, int64_t ldx, int64_t ldy, float eps);
+int32_t olmax_qk_rope_bwd(olmax_stream_t stream, const void* dy, void* dx, const void* x,
+                          const void* w, float* dw, const float* cos_t, const float* sin_t,
+                          int64_t tokens, int32_t heads, int32_t head_dim, int32_t seq_len,
+                          int64_t lddy, int64_t lddx, int64_t ldx, float eps);
+
+/* ---- Gated MLP activation: GatedMLP.forward, src/olmax/nn/mlp.py:69-73:
+ * out = act(gate) * up, act 0 = silu, 1 = tanh-approximated gelu (jax.nn.gelu default,
+ * src/olmax/nn/transformer/layer.py:133). */
+int32_t olmax_glu_fwd(olmax_stream_t stream, const void* gate, const void* up, void* out, int64_t T,
+                      int32_t F, int64_t ldg, int64_t ldu, int64_t ldo, int32_t act);
+int32_t olmax_glu_bwd(olmax_stream_t stream, const void* gate, const void* up, const void* dh,
+                      void* dgate, void* dup, int64_t T, int32_t F, int64_t ldg, int64_t ldu,
+                      int64_t lddh, int64_t lddg, int64_t lddu, int32_t act);
+
+/* ---- Attention: AttentionKernel.forward, src/olmax/nn/attention.py:52-109
+ * (jax.nn.dot_product_attention(is_causal=True, local_window_size=window)).
+ * BSHD: q [B*S, ldq] with head h at columns h*D.., k/v with KH heads (GQA: query head h reads
+ * kv head h / (H/KH)).  window < 0: global; window >= 0: keys i-window..i.  softcap > 0:
+ * scores <- softcap*tanh(scores/softcap) (extension, not in the reference).
+ * lse: fp32 [B, H, S], saved for the backward. */
+int32_t olmax_attn_fwd(olmax_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                       float* lse, int32_t B, int32_t S, int32_t H, int32_t KH, int32_t D, int64_t ldq,
+                       int64_t ldk, int64_t ldv, int64_t ldo, int32_t window, float softcap);
+int64_t olmax_attn_bwd_workspace_bytes(int32_t B, int32_t S, int32_t H, int32_t KH, int32_t D);
+int32_t olmax_attn_bwd(olmax_stream_t stream, const void* q, const void* k, const void* v,
+                       const void* o, const float* lse, const void* d_o, void* dq, void* dk, void* dv,
+                       void* workspace, int64_t workspace_bytes, int32_t B, int32_t S, int32_t H,
+                       int32_t KH, int32_t D, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo,
+                       int64_t lddo, int64_t lddq, int64_t lddk, int64_t lddv, int32_t window,
+                       float softcap);
+
+/* ---- Cross entropy: cross_entropy_loss / fused_cross_entropy_loss,
+ * src/olmax/nn/functional.py:70-121 (reduction "mean"; see the label quirks there).
+ * logits bf16 (logits_f32 == 0) or fp32; dlogits (optional, may alias logits) receives
+ * dloss * d loss / d logits; lse_out (optional [T]) the log-normaliser * (label != ignore). */
+int64_t olmax_cross_entropy_workspace_bytes(int64_t T);
+int32_t olmax_cross_entropy(olmax_stream_t stream, const void* logits, void* dlogits,
+                            const int32_t* labels, float* loss, float* lse_out, void* workspace,
+                            int64_t workspace_bytes, int64_t T, int32_t V, int64_t ld, int64_t ldd,
+                            int32_t logits_f32, int32_t ignore_index, float softcap, float dloss);
+
+/* ---- Fused LM head + cross entropy, forward and backward: LMHead.forward,
+ * src/olmax/nn/lm_head.py:59-61, followed by cross_entropy_loss as in the benchmark's
+ * loss_fun, src/integration_tests/train_transformer.py:190-206.
+ * dh / dW may be NULL to skip.  dw_f32 != 0: dW is fp32. */
+int64_t olmax_lmhead_ce_workspace_bytes(int64_t T, int32_t V);
+int32_t olmax_lmhead_ce(olmax_stream_t stream, const void* h, const void* W, const int32_t* labels,
+                        float* loss, void* dh, void* dW, void* workspace, int64_t workspace_bytes,
+                        int64_t T, int32_t d, int32_t V, int32_t ignore_index, float softcap,
+                        int32_t dw_f32);
+
+/* ---- Embedding: Embedding.forward, src/olmax/nn/embedding.py:30-32 (row gather) and its
+ * transpose (scatter-add; dW fp32 is ACCUMULATED into). */
+int32_t olmax_embed_fwd(olmax_stream_t stream, const int32_t* ids, const void* W, void* out, int64_t T,
+                        int32_t d, int32_t V);
+int32_t olmax_embed_bwd(olmax_stream_t stream, const int32_t* ids, const void* dh, float* dW, int64_t T,
+                        int32_t d, int32_t V);
+
+/* ---- AdamW: optax.adamw as built by AdamWConfig.build, src/olmax/optim/config.py:136-156,
+ * applied with eqx.apply_updates at src/olmax/train/trainer.py:745-752.  In place on fp32
+ * p/m/v; g bf16 or fp32 (scaled by grad_scale first: global-norm clipping,
+ * src/olmax/optim/utils.py:22-38); `step` is the 1-based count; shadow_bf16 (optional)
+ * receives bf16(p_new), replacing cast_tree(params, bf16) of trainer.py:728. */
+int32_t olmax_adamw(olmax_stream_t stream, float* p, const void* g, float* m, float* v,
+                    void* shadow_bf16, int64_t n, int32_t grad_is_bf16, float lr, float b1, float b2,
+                    float eps, float wd, int64_t step, float grad_scale);
+/* As olmax_adamw with an extra device-resident multiplier of the gradient (NULL = none). */
+int32_t olmax_adamw_dscale(olmax_stream_t stream, float* p, const void* g, float* m, float* v,
+                           void* shadow_bf16, int64_t n, int32_t grad_is_bf16, float lr, float b1,
+                           float b2, float eps, float wd, int64_t step, float grad_scale,
+                           const float* grad_scale_dev);
+/* *out += sum(g^2): building block of get_global_norm, src/olmax/jax_utils.py:88-102. */
+int32_t olmax_sumsq(olmax_stream_t stream, const void* g, int64_t n, int32_t is_bf16, float* out);
+
+/* ---- utilities */
+int32_t olmax_cast_f32_to_bf16(olmax_stream_t stream, const float* in, void* out, int64_t n);
+int32_t olmax_cast_bf16_to_f32(olmax_stream_t stream, const void* in, float* out, int64_t n);
+int32_t olmax_fill_zero(olmax_stream_t stream, void* p, int64_t nbytes);
+int32_t olmax_add_bf16(olmax_stream_t stream, const void* a, const void* b, void* out, int64_t n);
+
+/* =====================================================================================
+ * Whole block / whole model: the granularity Transformer.forward
+ * (src/olmax/nn/transformer/model.py:95-136) and process_microbatch
+ * (src/olmax/train/trainer.py:759-777) run at.
+ * ===================================================================================== */
+typedef struct {
+  int32_t vocab, d_model, n_layers, n_heads, n_kv_heads, head_dim, hidden;
+  int32_t layer_type; /* 0 TransformerLayer (pre-norm, layer.py:80-94), 1 ReorderedNorm
+                         (layer.py:102-116), 2 Gemma pre+post (layer.py:169-185) */
+  int32_t act;        /* 0 silu, 1 gelu-tanh */
+  int32_t qk_norm;    /* head-wise QK-norm (attention.py:293-296) */
+  int32_t tied;       /* LM head shares the embedding matrix (extension) */
+  int32_t batch, seq_len;
+  int32_t checkpoint; /* 1: full-block activation checkpointing (NothingSaveable,
+                         src/olmax/activation_checkpointing.py:71-80); 0: keep activations */
+  float eps, attn_softcap, final_softcap;
+} olmax_model_config;
+
+/* One parameter leaf inside the flat parameter buffer. */
+typedef struct {
+  int32_t kind;   /* OLMAX_LEAF_* */
+  int32_t layer;  /* -1 for global leaves */
+  int64_t offset; /* element offset in the flat fp32 master / bf16 working / bf16 grad buffers */
+  int64_t numel;
+  int32_t rows, cols;
+  int32_t grad_f32;     /* 1: gradient lives in the fp32 grad buffer at grad_f32_offset */
+  int64_t grad_f32_offset;
+} olmax_leaf;
+
+enum {
+  OLMAX_LEAF_EMBEDDING = 0, OLMAX_LEAF_Q, OLMAX_LEAF_K, OLMAX_LEAF_V, OLMAX_LEAF_O,
+  OLMAX_LEAF_GATE, OLMAX_LEAF_UP, OLMAX_LEAF_DOWN, OLMAX_LEAF_ATTN_NORM, OLMAX_LEAF_MLP_NORM,
+  OLMAX_LEAF_ATTN_IN_NORM, OLMAX_LEAF_MLP_IN_NORM, OLMAX_LEAF_Q_NORM, OLMAX_LEAF_K_NORM,
+  OLMAX_LEAF_FINAL_NORM, OLMAX_LEAF_LM_HEAD
+};
+
+/* Host-only layout queries. */
+int64_t olmax_model_num_params(const olmax_model_config* cfg);
+int64_t olmax_model_grad_f32_elems(const olmax_model_config* cfg);
+int32_t olmax_model_layout(const olmax_model_config* cfg, olmax_leaf* out, int32_t max_leaves);
+int64_t olmax_model_workspace_bytes(const olmax_model_config* cfg);
+
+/* loss + all gradients of one micro-batch: compute_loss_and_grads,
+ * src/olmax/train/trainer.py:723-740.
+ * params_bf16: flat bf16 working copy; ids/labels int32 [batch*seq_len];
+ * windows: host array [n_layers] (-1 = global); cos/sin: host arrays of n_layers device
+ * pointers to fp32 [seq_len, head_dim/2] tables (per-layer RoPE theta);
+ * grad_bf16 (flat, same offsets as params) and grad_f32 receive the gradients; loss: device
+ * fp32 scalar. */
+int32_t olmax_model_loss_and_grads(olmax_stream_t stream, const olmax_model_config* cfg,
+                                   const int32_t* windows, const float* const* cos_tables,
+                                   const float* const* sin_tables, const void* params_bf16,
+                                   const int32_t* ids, const int32_t* labels, float* loss,
+                                   void* grad_bf16, float* grad_f32, void* workspace,
+                                   int64_t workspace_bytes);
+/* Forward only (loss). */
+int32_t olmax_model_loss(olmax_stream_t stream, const olmax_model_config* cfg, const int32_t* windows,
+                         const float* const* cos_tables, const float* const* sin_tables,
+                         const void* params_bf16, const int32_t* ids, const int32_t* labels,
+                         float* loss, void* workspace, int64_t workspace_bytes);
+
+/* step_optimizer, src/olmax/train/trainer.py:742-757: fused AdamW over every leaf.
+ * decay_embedding == 0 masks "embedding.weight" from weight decay as the benchmark does
+ * (src/integration_tests/train_transformer.py:388).  max_grad_norm > 0 applies
+ * clip_grads_by_global_norm (src/olmax/optim/utils.py:22-38); norm_scratch: device float[2], left holding
+ * {clip factor, gradient norm}. */
+int32_t olmax_model_adamw(olmax_stream_t stream, const olmax_model_config* cfg, float* master,
+                          float* m, float* v, void* params_bf16, const void* grad_bf16,
+                          const float* grad_f32, int64_t step, float lr, float b1, float b2, float eps,
+                          float wd, int32_t decay_embedding, float max_grad_norm, float* norm_scratch);
+
+/* Single transformer block in isolation (any of the three orderings). */
+typedef struct {
+  const void *wqkv, *wo, *wgu, *wdown;          /* bf16: [(H+2K)D, d], [d, HD], [2F, d], [d, F] */
+  const void *attn_norm, *mlp_norm;             /* bf16 [d] */
+  const void *attn_in_norm, *mlp_in_norm;       /* bf16 [d], Gemma only */
+  const void *q_norm, *k_norm;                  /* bf16 [D], qk_norm only */
+} olmax_block_weights;
+typedef struct {
+  void *wqkv, *wo, *wgu, *wdown;                /* bf16, overwritten */
+  float *attn_norm, *mlp_norm, *attn_in_norm, *mlp_in_norm, *q_norm, *k_norm; /* fp32, accumulated */
+} olmax_block_grads;
+int64_t olmax_block_acts_bytes(const olmax_model_config* cfg);
+int64_t olmax_block_tmp_bytes(const olmax_model_config* cfg);
+int32_t olmax_block_fwd(olmax_stream_t stream, const olmax_model_config* cfg, const olmax_block_weights* w,
+                        int32_t window, const float* cos_t, const float* sin_t, const void* x, void* y,
+                        void* acts, int64_t acts_bytes);
+int32_t olmax_block_bwd(olmax_stream_t stream, const olmax_model_config* cfg, const olmax_block_weights* w,
+                        const olmax_block_grads* g, int32_t window, const float* cos_t,
+                        const float* sin_t, const void* x, const void* dy, void* dx, void* acts,
+                        int64_t acts_bytes, void* tmp, int64_t tmp_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OLMAX_HIP_H */

@@ -148,7 +148,9 @@ __global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ p, const
                                                     float* __restrict__ m, float* __restrict__ v,
                                                     bf16* __restrict__ shadow, int64_t n, float lr,
                                                     float b1, float b2, float eps, float wd,
-                                                    float bc1, float bc2, float gscale) {
+                                                    float bc1, float bc2, float gscale,
+                                                    const float* __restrict__ gscale_dev) {
+  if (gscale_dev) gscale *= *gscale_dev;
   const int64_t n4 = n / 4;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
     f32x4 pv = reinterpret_cast<const f32x4*>(p)[i];
@@ -313,9 +315,12 @@ extern "C" int32_t olmax_embed_bwd(hipStream_t stream, const int32_t* ids, const
   return OLMAX_OK;
 }
 
-extern "C" int32_t olmax_adamw(hipStream_t stream, float* p, const void* g, float* m, float* v,
-                               void* shadow_bf16, int64_t n, int32_t grad_is_bf16, float lr, float b1,
-                               float b2, float eps, float wd, int64_t step, float grad_scale) {
+// As olmax_adamw, with an additional device-resident gradient scale (NULL = none) so that
+// global-norm clipping needs no host round trip.
+extern "C" int32_t olmax_adamw_dscale(hipStream_t stream, float* p, const void* g, float* m, float* v,
+                                      void* shadow_bf16, int64_t n, int32_t grad_is_bf16, float lr, float b1,
+                                      float b2, float eps, float wd, int64_t step, float grad_scale,
+                                      const float* grad_scale_dev) {
   if (n == 0) return OLMAX_OK;
   OLMAX_CHECK(p && g && m && v, OLMAX_ERR_ARG, "olmax_adamw: null pointer");
   OLMAX_CHECK(n >= 0 && step >= 1, OLMAX_ERR_ARG, "olmax_adamw: n must be >= 0 and step >= 1 (1-based)");
@@ -326,11 +331,17 @@ extern "C" int32_t olmax_adamw(hipStream_t stream, float* p, const void* g, floa
   const float bc2 = (float)(1.0 - pow((double)b2, (double)step));
   const int grid = grid_1d((n + 3) / 4, 16384);
   if (grad_is_bf16)
-    hipLaunchKernelGGL(adamw_kernel<true>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale);
+    hipLaunchKernelGGL(adamw_kernel<true>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale, grad_scale_dev);
   else
-    hipLaunchKernelGGL(adamw_kernel<false>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale);
+    hipLaunchKernelGGL(adamw_kernel<false>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale, grad_scale_dev);
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
+}
+
+extern "C" int32_t olmax_adamw(hipStream_t stream, float* p, const void* g, float* m, float* v,
+                               void* shadow_bf16, int64_t n, int32_t grad_is_bf16, float lr, float b1,
+                               float b2, float eps, float wd, int64_t step, float grad_scale) {
+  return olmax_adamw_dscale(stream, p, g, m, v, shadow_bf16, n, grad_is_bf16, lr, b1, b2, eps, wd, step, grad_scale, nullptr);
 }
 
 // *out (fp32 scalar) += sum(g^2); the caller zeroes it.

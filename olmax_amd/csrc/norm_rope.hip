@@ -16,8 +16,10 @@ namespace {
 template <int LPR, int MAXC>
 __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16* __restrict__ x,
                                                           const bf16* __restrict__ w,
+                                                          const bf16* __restrict__ res,
                                                           bf16* __restrict__ y, int64_t rows, int d,
-                                                          int64_t ldx, int64_t ldy, float eps) {
+                                                          int64_t ldx, int64_t ldres, int64_t ldy,
+                                                          float eps) {
   constexpr int RPB = 256 / LPR;
   const int sub = threadIdx.x % LPR;
   const int rloc = threadIdx.x / LPR;
@@ -42,12 +44,14 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16* __restrict
 #pragma unroll
     for (int i = 0; i < MAXC; i++)
       if ((i * LPR + sub) * 8 < d) {
-        Pack8 wv, o;
+        Pack8 wv, rv, o;
         if (w) wv.u = *reinterpret_cast<const u32x4*>(w + (i * LPR + sub) * 8);
+        if (res) rv.u = *reinterpret_cast<const u32x4*>(res + row * ldres + (i * LPR + sub) * 8);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
           float v = r * bf2f(c[i].e[e]);
           if (w) v = bf2f(wv.e[e]) * v;
+          if (res) v = bf2f(f2bf(v)) + bf2f(rv.e[e]);  // the reference adds two bf16 arrays
           o.e[e] = f2bf(v);
         }
         *reinterpret_cast<u32x4*>(yr + (i * LPR + sub) * 8) = o.u;
@@ -58,8 +62,10 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16* __restrict
 // Any d (scalar accesses, one block per row): used for odd row lengths.
 __global__ __launch_bounds__(256) void rmsnorm_fwd_generic(const bf16* __restrict__ x,
                                                            const bf16* __restrict__ w,
+                                                           const bf16* __restrict__ res,
                                                            bf16* __restrict__ y, int64_t rows, int d,
-                                                           int64_t ldx, int64_t ldy, float eps) {
+                                                           int64_t ldx, int64_t ldres, int64_t ldy,
+                                                           float eps) {
   __shared__ float red[4];
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const bf16* xr = x + row * ldx;
@@ -73,6 +79,7 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_generic(const bf16* __restric
     for (int i = threadIdx.x; i < d; i += 256) {
       float v = r * bf2f(xr[i]);
       if (w) v = bf2f(w[i]) * v;
+      if (res) v = bf2f(f2bf(v)) + bf2f(res[row * ldres + i]);
       y[row * ldy + i] = f2bf(v);
     }
     __syncthreads();
@@ -310,22 +317,92 @@ __global__ __launch_bounds__(256) void qk_rope_bwd_kernel(
   }
 }
 
-// Any head_dim (even), scalar: one thread per rotation pair.  No norm fusion.
-__global__ void rope_generic_kernel(const bf16* __restrict__ x, bf16* __restrict__ y,
-                                    const float* __restrict__ cos_t,
-                                    const float* __restrict__ sin_t, int64_t tokens, int heads,
-                                    int D, int seq_len, int64_t ldx, int64_t ldy, float dir) {
-  const int half = D / 2;
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= tokens * heads * half) return;
-  const int i = (int)(idx % half);
-  const int h = (int)((idx / half) % heads);
-  const int64_t tok = idx / ((int64_t)half * heads);
+// Any even head_dim <= 512, strided views: one wave per (token, head); lane i handles rotation
+// pairs (i, i + D/2), (i + 64, ...).  Optional fused head-wise norm, same rounding as above.
+__global__ __launch_bounds__(64) void qk_rope_fwd_generic(
+    const bf16* __restrict__ x, bf16* __restrict__ y, const bf16* __restrict__ w,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int64_t tokens, int heads, int D,
+    int seq_len, int64_t ldx, int64_t ldy, float eps) {
+  const int64_t unit = blockIdx.x;
+  const int64_t tok = unit / heads;
+  const int h = (int)(unit % heads);
   const int pos = (int)(tok % seq_len);
-  const float cs = cos_t[(int64_t)pos * half + i], sn = dir * sin_t[(int64_t)pos * half + i];
-  const float a = bf2f(x[tok * ldx + h * D + i]), b = bf2f(x[tok * ldx + h * D + half + i]);
-  y[tok * ldy + h * D + i] = f2bf(a * cs - b * sn);
-  y[tok * ldy + h * D + half + i] = f2bf(b * cs + a * sn);
+  const int half = D / 2;
+  const bf16* xr = x + tok * ldx + h * D;
+  bf16* yr = y + tok * ldy + h * D;
+  float r = 1.f;
+  if (w) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < D; i += 64) {
+      const float f = bf2f(xr[i]);
+      ss += f * f;
+    }
+    ss = wave_sum(ss);
+    r = rsqrtf(ss / (float)D + eps);
+  }
+  for (int i = threadIdx.x; i < half; i += 64) {
+    float a = bf2f(xr[i]), b = bf2f(xr[i + half]);
+    if (w) {
+      a = bf2f(f2bf(bf2f(w[i]) * (r * a)));
+      b = bf2f(f2bf(bf2f(w[i + half]) * (r * b)));
+    }
+    const float cs = cos_t[(int64_t)pos * half + i], sn = sin_t[(int64_t)pos * half + i];
+    yr[i] = f2bf(a * cs - b * sn);
+    yr[i + half] = f2bf(b * cs + a * sn);
+  }
+}
+
+__global__ __launch_bounds__(64) void qk_rope_bwd_generic(
+    const bf16* __restrict__ dy, bf16* __restrict__ dx, const bf16* __restrict__ x,
+    const bf16* __restrict__ w, float* __restrict__ dw, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int64_t tokens, int heads, int D, int seq_len, int64_t lddy,
+    int64_t lddx, int64_t ldx, float eps) {
+  const int64_t unit = blockIdx.x;
+  const int64_t tok = unit / heads;
+  const int h = (int)(unit % heads);
+  const int pos = (int)(tok % seq_len);
+  const int half = D / 2;
+  const bf16* dyr = dy + tok * lddy + h * D;
+  bf16* dxr = dx + tok * lddx + h * D;
+  // each lane owns pairs i = lane, lane+64, ... (at most 4 pairs for D <= 512)
+  float ga[4], gb[4];
+  int np = 0;
+  for (int i = threadIdx.x; i < half; i += 64, np++) {
+    const float d1 = bf2f(dyr[i]), d2 = bf2f(dyr[i + half]);
+    const float cs = cos_t[(int64_t)pos * half + i], sn = sin_t[(int64_t)pos * half + i];
+    ga[np] = d1 * cs + d2 * sn;
+    gb[np] = d2 * cs - d1 * sn;
+  }
+  if (!w) {
+    np = 0;
+    for (int i = threadIdx.x; i < half; i += 64, np++) {
+      dxr[i] = f2bf(ga[np]);
+      dxr[i + half] = f2bf(gb[np]);
+    }
+    return;
+  }
+  const bf16* xr = x + tok * ldx + h * D;
+  float ss = 0.f, sxg = 0.f;
+  np = 0;
+  for (int i = threadIdx.x; i < half; i += 64, np++) {
+    ga[np] = bf2f(f2bf(ga[np]));
+    gb[np] = bf2f(f2bf(gb[np]));
+    const float xa = bf2f(xr[i]), xb = bf2f(xr[i + half]);
+    ss += xa * xa + xb * xb;
+    sxg += xa * bf2f(w[i]) * ga[np] + xb * bf2f(w[i + half]) * gb[np];
+  }
+  ss = wave_sum(ss);
+  sxg = wave_sum(sxg);
+  const float r = rsqrtf(ss / (float)D + eps);
+  const float coef = r * r * r * (sxg / (float)D);
+  np = 0;
+  for (int i = threadIdx.x; i < half; i += 64, np++) {
+    const float xa = bf2f(xr[i]), xb = bf2f(xr[i + half]);
+    dxr[i] = f2bf(r * bf2f(w[i]) * ga[np] - xa * coef);
+    dxr[i + half] = f2bf(r * bf2f(w[i + half]) * gb[np] - xb * coef);
+    atomicAdd(&dw[i], ga[np] * xa * r);
+    atomicAdd(&dw[i + half], gb[np] * xb * r);
+  }
 }
 
 int grid_for(int64_t work_items, int per_block, int cap) {
@@ -337,25 +414,34 @@ int grid_for(int64_t work_items, int per_block, int cap) {
 
 }  // namespace
 
-extern "C" int32_t olmax_rmsnorm_fwd(hipStream_t stream, const void* x, const void* w, void* y,
-                                     int64_t rows, int32_t d, int64_t ldx, int64_t ldy, float eps) {
+// y = rms_norm(x, w) (+ res): res (optional, bf16 [rows, d]) is the residual stream added after
+// the normalised value has been rounded to bf16 (post-norm layers: h = x + norm(f(x))).
+extern "C" int32_t olmax_rmsnorm_fwd_res(hipStream_t stream, const void* x, const void* w,
+                                         const void* res, void* y, int64_t rows, int32_t d,
+                                         int64_t ldx, int64_t ldres, int64_t ldy, float eps) {
   if (rows == 0) return OLMAX_OK;
   OLMAX_CHECK(x && y, OLMAX_ERR_ARG, "olmax_rmsnorm_fwd: null pointer");
-  OLMAX_CHECK(rows >= 0 && d > 0 && ldx >= d && ldy >= d, OLMAX_ERR_SHAPE, "olmax_rmsnorm_fwd: bad shape rows=%ld d=%d", (long)rows, d);
-  const bool vec = aligned16(x) && aligned16(y) && (!w || aligned16(w)) && ldx % 8 == 0 && ldy % 8 == 0;
-  const bf16 *xp = (const bf16*)x, *wp = (const bf16*)w;
+  OLMAX_CHECK(rows >= 0 && d > 0 && ldx >= d && ldy >= d && (!res || ldres >= d), OLMAX_ERR_SHAPE, "olmax_rmsnorm_fwd: bad shape rows=%ld d=%d", (long)rows, d);
+  const bool vec = aligned16(x) && aligned16(y) && (!w || aligned16(w)) && ldx % 8 == 0 && ldy % 8 == 0 &&
+                   (!res || (aligned16(res) && ldres % 8 == 0));
+  const bf16 *xp = (const bf16*)x, *wp = (const bf16*)w, *rp = (const bf16*)res;
   bf16* yp = (bf16*)y;
   if (vec && d % 8 == 0 && d <= 256) {
-    hipLaunchKernelGGL((rmsnorm_fwd_kernel<16, 2>), dim3(grid_for(rows, 16, 1 << 20)), dim3(256), 0, stream, xp, wp, yp, rows, d, ldx, ldy, eps);
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<16, 2>), dim3(grid_for(rows, 16, 1 << 20)), dim3(256), 0, stream, xp, wp, rp, yp, rows, d, ldx, ldres, ldy, eps);
   } else if (vec && d % 8 == 0 && d <= 4096) {
-    hipLaunchKernelGGL((rmsnorm_fwd_kernel<64, 8>), dim3(grid_for(rows, 4, 1 << 20)), dim3(256), 0, stream, xp, wp, yp, rows, d, ldx, ldy, eps);
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<64, 8>), dim3(grid_for(rows, 4, 1 << 20)), dim3(256), 0, stream, xp, wp, rp, yp, rows, d, ldx, ldres, ldy, eps);
   } else if (vec && d % 8 == 0 && d <= 8192) {
-    hipLaunchKernelGGL((rmsnorm_fwd_kernel<64, 16>), dim3(grid_for(rows, 4, 1 << 20)), dim3(256), 0, stream, xp, wp, yp, rows, d, ldx, ldy, eps);
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<64, 16>), dim3(grid_for(rows, 4, 1 << 20)), dim3(256), 0, stream, xp, wp, rp, yp, rows, d, ldx, ldres, ldy, eps);
   } else {
-    hipLaunchKernelGGL(rmsnorm_fwd_generic, dim3(grid_for(rows, 1, 1 << 16)), dim3(256), 0, stream, xp, wp, yp, rows, d, ldx, ldy, eps);
+    hipLaunchKernelGGL(rmsnorm_fwd_generic, dim3(grid_for(rows, 1, 1 << 16)), dim3(256), 0, stream, xp, wp, rp, yp, rows, d, ldx, ldres, ldy, eps);
   }
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
+}
+
+extern "C" int32_t olmax_rmsnorm_fwd(hipStream_t stream, const void* x, const void* w, void* y,
+                                     int64_t rows, int32_t d, int64_t ldx, int64_t ldy, float eps) {
+  return olmax_rmsnorm_fwd_res(stream, x, w, nullptr, y, rows, d, ldx, 0, ldy, eps);
 }
 
 // dw (fp32, [d]) is ACCUMULATED into: the caller zeroes it.  dres (optional) is added to dx.
@@ -405,19 +491,8 @@ extern "C" int32_t olmax_qk_rope_fwd(hipStream_t stream, const void* x, void* y,
     else
       hipLaunchKernelGGL(qk_rope_fwd_kernel<false>, grid, dim3(256), 0, stream, xp, yp, (const bf16*)nullptr, cos_t, sin_t, tokens, heads, seq_len, ldx, ldy, eps);
   } else {
-    const bf16* src = xp;
-    int64_t lds = ldx;
-    if (w) {  // unfused: norm over rows of head_dim, then rotate in place
-      // rows of one token are contiguous heads: treat [tokens, heads, D] with row stride D only
-      // when the view is dense; otherwise norm token by token is not expressible -> reject.
-      OLMAX_CHECK(ldx == (int64_t)heads * head_dim && ldy == ldx, OLMAX_ERR_SHAPE, "olmax_qk_rope_fwd: strided views need head_dim == 128 when the norm is fused");
-      int rc = olmax_rmsnorm_fwd(stream, x, w, y, tokens * heads, head_dim, head_dim, head_dim, eps);
-      if (rc) return rc;
-      src = yp;
-      lds = ldy;
-    }
-    const int64_t n = tokens * heads * (head_dim / 2);
-    hipLaunchKernelGGL(rope_generic_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, src, yp, cos_t, sin_t, tokens, heads, head_dim, seq_len, lds, ldy, 1.f);
+    OLMAX_CHECK(head_dim <= 512, OLMAX_ERR_SHAPE, "olmax_qk_rope_fwd: head_dim > 512 unsupported");
+    hipLaunchKernelGGL(qk_rope_fwd_generic, dim3((unsigned)(tokens * heads)), dim3(64), 0, stream, xp, yp, (const bf16*)w, cos_t, sin_t, tokens, heads, head_dim, seq_len, ldx, ldy, eps);
   }
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
@@ -444,13 +519,8 @@ extern "C" int32_t olmax_qk_rope_bwd(hipStream_t stream, const void* dy, void* d
     else
       hipLaunchKernelGGL(qk_rope_bwd_kernel<false>, grid, dim3(256), 0, stream, dyp, dxp, (const bf16*)nullptr, (const bf16*)nullptr, (float*)nullptr, cos_t, sin_t, tokens, heads, seq_len, lddy, lddx, ldx, eps);
   } else {
-    const int64_t n = tokens * heads * (head_dim / 2);
-    hipLaunchKernelGGL(rope_generic_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, dyp, dxp, cos_t, sin_t, tokens, heads, head_dim, seq_len, lddy, lddx, -1.f);
-    if (w) {
-      OLMAX_CHECK(lddx == (int64_t)heads * head_dim && ldx == lddx, OLMAX_ERR_SHAPE, "olmax_qk_rope_bwd: strided views need head_dim == 128 when the norm is fused");
-      int rc = olmax_rmsnorm_bwd(stream, x, w, dx, nullptr, dx, dw, tokens * heads, head_dim, head_dim, head_dim, 0, head_dim, eps);
-      if (rc) return rc;
-    }
+    OLMAX_CHECK(head_dim <= 512, OLMAX_ERR_SHAPE, "olmax_qk_rope_bwd: head_dim > 512 unsupported");
+    hipLaunchKernelGGL(qk_rope_bwd_generic, dim3((unsigned)(tokens * heads)), dim3(64), 0, stream, dyp, dxp, (const bf16*)x, (const bf16*)w, dw, cos_t, sin_t, tokens, heads, head_dim, seq_len, lddy, lddx, ldx, eps);
   }
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;

@@ -394,7 +394,7 @@ def init_params(cfg: ModelConfig, seed: int = 0, std: float = 0.02, dtype=torch.
             p[pre + "mlp_input_norm.weight"] = torch.ones(d, dtype=dtype)
     p["norm.weight"] = torch.ones(d, dtype=dtype)
     if not cfg.tied:
-        p["lm_head.w_out.weight"] = n(cfg.vocab, d)
+        p["lm_head.proj.weight"] = n(cfg.vocab, d)
     return p
 
 
@@ -529,7 +529,7 @@ def model_loss_and_grads(cfg: ModelConfig, P: dict, ids: Tensor, labels: Tensor,
         h, tape = block_fwd(cfg, P, l, h, rt)
         tapes.append(tape)
     hn = rms_norm_fwd(h, P["norm.weight"], cfg.eps, rt)
-    w_out = P["embedding.weight"] if cfg.tied else P["lm_head.w_out.weight"]
+    w_out = P["embedding.weight"] if cfg.tied else P["lm_head.proj.weight"]
     B, S, d = hn.shape
     loss, dhn, dw_out = lm_head_ce(hn.reshape(B * S, d), w_out, labels.reshape(-1),
                                    softcap=cfg.final_softcap, rt=rt)
@@ -541,7 +541,7 @@ def model_loss_and_grads(cfg: ModelConfig, P: dict, ids: Tensor, labels: Tensor,
         G["embedding.weight"] = rt(demb + dw_out)
     else:
         G["embedding.weight"] = rt(demb)
-        G["lm_head.w_out.weight"] = dw_out
+        G["lm_head.proj.weight"] = dw_out
     return loss, G
 
 

@@ -245,7 +245,7 @@ def _autograd_model_loss(cfg, P, ids, labels):
     for l in range(cfg.n_layers):
         h, _ = ref.block_fwd(cfg, P, l, h)
     hn = ref.rms_norm_fwd(h, P["norm.weight"], cfg.eps)
-    w = P["embedding.weight"] if cfg.tied else P["lm_head.w_out.weight"]
+    w = P["embedding.weight"] if cfg.tied else P["lm_head.proj.weight"]
     logits = hn @ w.t()
     return ref.cross_entropy_fwd(logits.reshape(-1, cfg.vocab), labels.reshape(-1), softcap=cfg.final_softcap)[0]
 
