@@ -1,0 +1,160 @@
+#!/usr/bin/env python3
+"""Benchmark of the HIP train step: Llama-like 7B, seq 4096, micro-batch 2, bf16 compute,
+fp32 master weights + AdamW, full-block activation checkpointing, one MI355X.
+
+Prints ONE JSON line: whole-job train tokens/s (inputs resident in HBM), bf16 MFU, the
+roofline figures of the dominant kernel (the bf16 MFMA GEMM, timed live with HIP events on
+its launch stream) and a CPU baseline (the CPU oracle, "port") on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16 = 2.5e15  # dense MFMA bf16 FLOP/s of one MI355X
+
+
+def cpu_baseline(sample_tokens: int = 512):
+    """CPU oracle timed on a bounded sample of the SAME workload: one of the 32 blocks of the 7B
+    model (d 4096, 32x128 heads, hidden 11008) forward + backward + AdamW on `sample_tokens`
+    tokens of one sequence, plus the LM head + cross entropy (vocab 100352) on those tokens,
+    fp32, all host threads.  Extrapolated to the full step: 32 x block + head."""
+    import torch
+    from oracle import ref
+
+    cfg = ref.ModelConfig(vocab=100352, d_model=4096, n_layers=1, n_heads=32, n_kv_heads=32, head_dim=128,
+                          hidden=11008, eps=1e-6, rope_theta=5e5)
+    g = torch.Generator().manual_seed(0)
+    P = {k: v for k, v in ref.init_params(cfg, seed=0).items() if k.startswith("layers.0.")}
+    x = torch.randn(1, sample_tokens, 4096, generator=g)
+    dy = torch.randn(1, sample_tokens, 4096, generator=g)
+    G = {}
+    t0 = time.perf_counter()
+    y, tape = ref.block_fwd(cfg, P, 0, x)
+    ref.block_bwd(cfg, P, 0, dy, tape, G)
+    for n in P:
+        ref.adamw_step(P[n], G[n], torch.zeros_like(P[n]), torch.zeros_like(P[n]), step=1, lr=1e-4)
+    t_block = time.perf_counter() - t0
+    W = torch.randn(100352, 4096, generator=g) * 0.02
+    labels = torch.randint(0, 100352, (sample_tokens,), generator=g)
+    t0 = time.perf_counter()
+    ref.lm_head_ce(x[0], W, labels)
+    t_head = time.perf_counter() - t0
+    est = 32 * t_block + t_head
+    return {
+        "value": sample_tokens / est, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"1 of 32 blocks fwd+bwd+AdamW ({t_block:.2f} s) + LM head/CE fwd+bwd ({t_head:.2f} s) on "
+                  f"{sample_tokens} tokens of one sequence, fp32 torch-CPU oracle; step time extrapolated as "
+                  f"32 x block + head (no recompute, attention over {sample_tokens} keys only)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--no-checkpoint", action="store_true", help="keep activations instead of full-block recompute")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline metric)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE MI355X only (no collectives or sharding); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from olmax_amd import AdamWConfig, Trainer, TransformerRecipe, WarmupCosineDecaySchedule, _lib
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    L = _lib.load()
+    B, S = 2, 4096
+    cfg = TransformerRecipe.llama_like_7B_bench()
+    cfg.num_layers = args.layers
+    if args.no_checkpoint:
+        cfg.layer_ac_policy = None
+    model = cfg.build(batch_size=B, sequence_length=S, seed=0)
+    # the reference benchmark's optimizer: AdamW, cosine 1e-6 -> 1e-4 -> 1e-6, embedding not decayed
+    optim = AdamWConfig(lr=WarmupCosineDecaySchedule(warmup_steps=20, decay_steps=80, peak_value=1e-4,
+                                                     init_value=1e-6, end_value=1e-6),
+                        no_decay_modules=["embedding.weight"])
+    trainer = Trainer(model, optim)
+    T = B * S
+    nb = 4
+    gen = torch.Generator().manual_seed(0)
+    batches = []
+    for _ in range(nb):
+        ids = torch.randint(0, cfg.vocab_size, (T,), generator=gen, dtype=torch.int32).cuda()
+        labels = torch.randint(0, cfg.vocab_size, (T,), generator=gen, dtype=torch.int32).cuda()
+        batches.append((ids, labels))
+
+    losses = []
+    for i in range(args.warmup):
+        losses.append(trainer.process_microbatch(*batches[i % nb]))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        losses.append(trainer.process_microbatch(*batches[(args.warmup + i) % nb]))
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / max(1, args.steps) * 1e3
+    tps = T * args.steps / dt
+    flops_tok = cfg.flops_per_token(S)
+    mfu = tps * flops_tok / PEAK_BF16
+    losses = [float(l) if not hasattr(l, "item") else l.item() for l in losses[-1:]]
+
+    # ---- roofline of the dominant kernel: one more (untimed) step with a HIP-event pair around
+    # every GEMM launch, recorded on the launch stream
+    L.olmax_gemm_profile_begin()
+    trainer.process_microbatch(*batches[0])
+    torch.cuda.synchronize()
+    cap = 64
+    keys = (ctypes.c_int32 * cap)(); ms = (ctypes.c_double * cap)(); fl = (ctypes.c_double * cap)(); ln = (ctypes.c_int64 * cap)()
+    n = L.olmax_gemm_profile_end(keys, ms, fl, ln, cap)
+    per = []
+    for i in range(n):
+        k = keys[i]
+        name = "gemm_bf16_kernel<tile%d,%s,%s%s%s>" % (k & 0xfff, "A_KC" if k >> 12 & 1 else "A_MC", "B_KC" if k >> 13 & 1 else "B_NC",
+                                                       ",res" if k >> 14 & 1 else "", ",f32out" if k >> 15 & 1 else "")
+        per.append({"kernel": name, "launches": ln[i], "total_ms": ms[i], "avg_ms": ms[i] / ln[i], "tflops": fl[i] / ms[i] / 1e9})
+    per.sort(key=lambda r: -r["total_ms"])
+    dom = per[0] if per else None
+    gemm_ms = sum(r["total_ms"] for r in per)
+    gemm_fl = sum(r["tflops"] * r["total_ms"] for r in per)  # TFLOP*1e-3... (tflops * ms = GFLOP)
+    roofline = None
+    if dom:
+        roofline = {"bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s",
+                    "frac": dom["tflops"] / (PEAK_BF16 / 1e12), "traffic": None, "kernel": dom["kernel"],
+                    "avg_launch_ms": dom["avg_ms"], "launches_per_step": dom["launches"],
+                    "all_gemm": {"ms_per_step": gemm_ms, "tflops": gemm_fl / gemm_ms if gemm_ms else None,
+                                 "share_of_step": gemm_ms / ms_per_step}}
+
+    out = {
+        "metric": "train tokens/sec + bf16 MFU, Llama-like 7B seq 4096 mb=2, 1 MI355X",
+        "value": tps, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (uniform tokens, N(0,0.02) init, resident in HBM)",
+        "mfu_bf16": mfu, "gflop_per_token": flops_tok / 1e9, "last_loss": losses[-1],
+        "config": {"workload": "Llama-like 7B full train step (configs[2]): 32 layers, d_model 4096, 32x128 heads, "
+                               "SwiGLU 11008, vocab 100352 untied, seq 4096, micro-batch 2, bf16 compute, fp32 master + "
+                               "AdamW, " + ("activations kept (no recompute)" if args.no_checkpoint else "full-block activation checkpointing"),
+                   "layers": cfg.num_layers, "global_batch": B, "seq_len": S, "params": model.num_params,
+                   "activation_checkpointing": not args.no_checkpoint},
+        "roofline": roofline,
+        "gemm_kernels": per[:6],
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

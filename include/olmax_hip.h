@@ -47,6 +47,12 @@ int32_t olmax_gemm_bf16(olmax_stream_t stream, const void* A, const void* B, voi
                         int64_t ldr, int32_t a_layout, int32_t b_layout, int32_t out_f32);
 /* Test/tuning hook: force the MFMA tile variant (0 = automatic). */
 void olmax_gemm_set_tile(int tile);
+/* Diagnostic: record a HIP-event pair on the launch stream around every MFMA GEMM launch
+ * between begin and end (allocates events; not for graph capture).  end() waits for them and
+ * aggregates per kernel instantiation: key = tile | a_kc<<12 | b_kc<<13 | has_res<<14 |
+ * out_f32<<15.  Returns the number of distinct keys written (at most cap). */
+void olmax_gemm_profile_begin(void);
+int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, int64_t* launches, int32_t cap);
 
 /* ---- RMSNorm: rms_norm, src/olmax/nn/functional.py:51-67; RMSNorm.forward,
  * src/olmax/nn/normalization.py:85-87.  w may be NULL (no scale). */

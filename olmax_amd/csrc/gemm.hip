@@ -24,10 +24,23 @@
 // every XCD one contiguous run of tiles; runs walk the tile grid in column groups so that
 // the A row-panels and B column-panels a single L2 sees are re-used.
 #include "common.h"
+#include <vector>
+#include <mutex>
 
 namespace {
 
 constexpr int BK = 64;
+
+// Optional per-launch timing (HIP events recorded on the launch stream around every GEMM),
+// switched on by olmax_gemm_profile_begin(); used by the benchmark's roofline report.
+struct ProfRec {
+  hipEvent_t e0, e1;
+  double flops;
+  int key;  // tile | a_kc<<12 | b_kc<<13 | has_res<<14 | out_f32<<15
+};
+bool g_prof_on = false;
+std::vector<ProfRec> g_prof;
+std::mutex g_prof_mu;
 
 template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
@@ -268,8 +281,21 @@ int launch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16
     attr_set = true;
   }
   const int tm = M / BM, tn = N / BN;
+  ProfRec rec{};
+  if (g_prof_on) {
+    (void)hipEventCreate(&rec.e0);
+    (void)hipEventCreate(&rec.e1);
+    (void)hipEventRecord(rec.e0, s);
+  }
   hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(NT), SMEM, s, A, B, C, R, M, N, K, lda, ldb, ldc,
                      ldr, tm, tn);
+  if (g_prof_on) {
+    (void)hipEventRecord(rec.e1, s);
+    rec.flops = 2.0 * M * N * K;
+    rec.key = (BM == 256 ? (WN == 64 ? 256 : 257) : 128) | (A_KC << 12) | (B_KC << 13) | (HAS_RES << 14) | (OUT_F32 << 15);
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof.push_back(rec);
+  }
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
 }
@@ -292,6 +318,40 @@ int g_force_tile = 0;
 }  // namespace
 
 extern "C" void olmax_gemm_set_tile(int tile) { g_force_tile = tile; }
+
+// Start recording a HIP-event pair around every MFMA GEMM launch (diagnostic; allocates events).
+extern "C" void olmax_gemm_profile_begin(void) {
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  g_prof.clear();
+  g_prof_on = true;
+}
+// Stop recording, wait for the recorded events and aggregate per kernel instantiation.
+// keys/ms/flops/launches: host arrays of `cap` entries; returns the number of distinct keys.
+// key = tile | a_layout<<12 | b_layout<<13 | has_residual<<14 | out_f32<<15, with a_layout /
+// b_layout bit SET when the operand is reduction-contiguous.
+extern "C" int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, int64_t* launches, int32_t cap) {
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  g_prof_on = false;
+  int n = 0;
+  for (auto& r : g_prof) {
+    (void)hipEventSynchronize(r.e1);
+    float t = 0.f;
+    (void)hipEventElapsedTime(&t, r.e0, r.e1);
+    int i = 0;
+    for (; i < n; i++)
+      if (keys[i] == r.key) break;
+    if (i == n) {
+      if (n >= cap) continue;
+      keys[n] = r.key; ms[n] = 0; flops[n] = 0; launches[n] = 0;
+      n++;
+    }
+    ms[i] += t; flops[i] += r.flops; launches[i] += 1;
+    (void)hipEventDestroy(r.e0);
+    (void)hipEventDestroy(r.e1);
+  }
+  g_prof.clear();
+  return n;
+}
 
 extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void* B, void* C,
                                    const void* R, int32_t M, int32_t N, int32_t K, int64_t lda,
