@@ -26,6 +26,7 @@ FLAGS = [
     "-munsafe-fp-atomics",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
+    "-Wno-inline-asm",
     "-Wno-unknown-warning-option",
     "-I", str(CSRC),
     "-I", str(HERE.parent / "include"),

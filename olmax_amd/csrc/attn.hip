@@ -28,9 +28,11 @@ __device__ __forceinline__ float fexp2(float x) { return __builtin_amdgcn_exp2f(
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 
-// chunk swizzle: distinct over any 8 consecutive rows (b128 reads) and pair-distinct over
-// any aligned 4 consecutive rows (transposing b64 reads)
-__device__ __forceinline__ int swz(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
+// 16-byte chunk swizzle of the [rows][128] tiles (256 B rows = one line of the 64 LDS banks).
+// ds_read_b128 serves the lane groups {0-3,12-15,20-23,24-27} / {4-7,8-11,16-19,28-31} (one
+// row per lane, same logical chunk) per clock and the transposing ds_read_b64 serves lanes
+// 0-31 (4 consecutive rows x 4 chunks); this mask gives 16 distinct chunks in both cases.
+__device__ __forceinline__ int swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
 // byte offset of 16B chunk `c` (0..15) of row `row` in a [rows][128] bf16 tile
 __device__ __forceinline__ int tile_off(int row, int c) { return row * 256 + ((c ^ swz(row)) << 4); }

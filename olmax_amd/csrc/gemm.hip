@@ -12,12 +12,19 @@
 // dW = dY^T X             : A=dY (MC), B=X  (NC)   (reduction over tokens)
 //
 // Tiling: BM x BN x 64 block tile, 64-lane waves each owning a WM x WN sub-tile as
-// (WM/32) x (WN/32) v_mfma_f32_32x32x16_bf16 accumulators. Operand tiles are staged
-// through LDS with a register-held prefetch of the next k-tile (double buffered LDS,
-// one barrier per k-tile). K-contiguous tiles live in LDS as [rows][64] with the 16-byte
-// chunk index XOR-swizzled by row so ds_read_b128 is bank-conflict free; M/N-contiguous
+// (WM/32) x (WN/32) v_mfma_f32_32x32x16_bf16 accumulators. Operand tiles stream from
+// global memory straight into LDS (global_load_lds_dwordx4, no VGPR staging, no LDS-write
+// phase) into the stage that is not being consumed; one barrier per k-tile. K-contiguous tiles live in LDS as [rows][64]; M/N-contiguous
 // tiles live as [64][rows] and are read with ds_read_b64_tr_b16, the gfx950 transposing
 // LDS load, which hands each lane 4 consecutive reduction-dim elements of its column.
+//
+// LDS bank geometry (measured on gfx950 with SQ_LDS_BANK_CONFLICT): 64 banks x 4 B, i.e.
+// 256 B per clock.  ds_read_b128 serves 16 lanes per clock in the fixed groups
+// {0-3,12-15,20-23,24-27}, {4-7,8-11,16-19,28-31} (+32 for the upper half); ds_read_b64
+// serves lanes 0-31, then 32-63.  The 16-byte chunk index of every tile is XOR-swizzled so
+// that each such group touches 16 distinct chunks modulo 256 B:
+//   [rows][64]  (128 B rows, two rows per bank line): chunk ^= (row >> 1) & 7
+//   [64][rows]  (transposing reads cover 4 k-rows x 64 B): chunk ^= (k & 3) << 2
 //
 // Workgroup -> tile mapping is XCD aware: hardware deals consecutive workgroup ids
 // round-robin over the 8 XCDs, so id i is remapped to (i % 8) * (grid/8) + i / 8, giving
@@ -42,24 +49,33 @@ bool g_prof_on = false;
 std::vector<ProfRec> g_prof;
 std::mutex g_prof_mu;
 
+// 16 B per lane straight from global memory into LDS at (lds_addr + lane*16); lds_addr is
+// wave-uniform (it travels in M0).  Issued as inline asm so that the compiler does not
+// serialise later LDS reads behind it; completion is awaited explicitly (vmcnt) before the
+// barrier that publishes the tile.
+__device__ __forceinline__ void dma16(const void* g, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(g) : "m0", "memory");
+}
+
 template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
     const bf16* __restrict__ A, const bf16* __restrict__ B, void* __restrict__ Cv,
     const bf16* __restrict__ R, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
     int64_t ldr, int tiles_m, int tiles_n) {
-  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int WAVES_N = BN / WN;
-  constexpr int A_CHUNKS = BM * BK / 8 / NT;  // 16-byte chunks per thread per k-tile
-  constexpr int B_CHUNKS = BN * BK / 8 / NT;
-  static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "tile too small for thread count");
   constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+  constexpr int A_INS = A_BYTES / 1024 / NW;  // DMA instructions (1 KB each) per wave per k-tile
+  constexpr int B_INS = B_BYTES / 1024 / NW;
+  static_assert(A_INS >= 1 && B_INS >= 1, "tile too small for the wave count");
+  constexpr int NINS = A_INS + B_INS;
+  constexpr int STAGE = A_BYTES + B_BYTES;
 
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  // layout: [stage][A tile | B tile]
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [2 stages][A tile | B tile]
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
   // ---- XCD-aware tile assignment ----
@@ -79,43 +95,37 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
   const int tile_n = (pid % group_sz) / gm;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-  // ---- per-thread global source addresses ----
-  const bf16* a_src[A_CHUNKS];
-  int a_dst[A_CHUNKS];
+  // ---- per-lane DMA sources: instruction i of this wave fills LDS block (i*NW + wave) of
+  // 1 KB, i.e. 16-byte chunks p = block*64 + lane of the tile; the lane fetches whichever
+  // global chunk the swizzle places there ----
+  const bf16* a_src[A_INS];
 #pragma unroll
-  for (int i = 0; i < A_CHUNKS; i++) {
-    const int q = i * NT + tid;
+  for (int i = 0; i < A_INS; i++) {
+    const int p = (i * NW + wave) * 64 + lane;
     if (A_KC) {
-      const int row = q >> 3, kc = q & 7;
-      a_src[i] = A + (int64_t)(m0 + row) * lda + kc * 8;
-      a_dst[i] = row * 128 + ((kc ^ (row & 7)) << 4);
+      const int row = p >> 3, ph = p & 7;
+      a_src[i] = A + (int64_t)(m0 + row) * lda + ((ph ^ ((row >> 1) & 7)) << 3);
     } else {
       constexpr int CPR = BM / 8;  // chunks per k-row
-      const int kr = q / CPR, mc = q % CPR;
-      a_src[i] = A + (int64_t)kr * lda + m0 + mc * 8;
-      a_dst[i] = kr * (BM * 2) + ((mc ^ ((kr & 3) << 1)) << 4);
+      const int kr = p / CPR, ph = p % CPR;
+      a_src[i] = A + (int64_t)kr * lda + m0 + ((ph ^ ((kr & 3) << 2)) << 3);
     }
   }
-  const bf16* b_src[B_CHUNKS];
-  int b_dst[B_CHUNKS];
+  const bf16* b_src[B_INS];
 #pragma unroll
-  for (int i = 0; i < B_CHUNKS; i++) {
-    const int q = i * NT + tid;
+  for (int i = 0; i < B_INS; i++) {
+    const int p = (i * NW + wave) * 64 + lane;
     if (B_KC) {
-      const int row = q >> 3, kc = q & 7;
-      b_src[i] = B + (int64_t)(n0 + row) * ldb + kc * 8;
-      b_dst[i] = row * 128 + ((kc ^ (row & 7)) << 4);
+      const int row = p >> 3, ph = p & 7;
+      b_src[i] = B + (int64_t)(n0 + row) * ldb + ((ph ^ ((row >> 1) & 7)) << 3);
     } else {
       constexpr int CPR = BN / 8;
-      const int kr = q / CPR, nc = q % CPR;
-      b_src[i] = B + (int64_t)kr * ldb + n0 + nc * 8;
-      b_dst[i] = kr * (BN * 2) + ((nc ^ ((kr & 3) << 1)) << 4);
+      const int kr = p / CPR, ph = p % CPR;
+      b_src[i] = B + (int64_t)kr * ldb + n0 + ((ph ^ ((kr & 3) << 2)) << 3);
     }
   }
   const int64_t a_step = A_KC ? (int64_t)BK : (int64_t)BK * lda;
   const int64_t b_step = B_KC ? (int64_t)BK : (int64_t)BK * ldb;
-
-  u32x4 a_reg[A_CHUNKS], b_reg[B_CHUNKS];
 
   f32x16 acc[TM][TN];
 #pragma unroll
@@ -126,99 +136,103 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
   const int KT = K / BK;
-
-  auto gload = [&](int kt) {
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  // issue DMA instructions [lo, hi) of the combined A+B list of k-tile kt into `stage`
+  auto dma = [&](int kt, int stage, int lo, int hi) {
+    const unsigned sa = lds_base + stage * STAGE;
+    const unsigned sb = sa + A_BYTES;
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; i++)
-      a_reg[i] = *reinterpret_cast<const u32x4*>(a_src[i] + (int64_t)kt * a_step);
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; i++)
-      b_reg[i] = *reinterpret_cast<const u32x4*>(b_src[i] + (int64_t)kt * b_step);
-  };
-  auto lstore = [&](int stage) {
-    unsigned char* sa = smem + stage * (A_BYTES + B_BYTES);
-    unsigned char* sb = sa + A_BYTES;
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; i++) *reinterpret_cast<u32x4*>(sa + a_dst[i]) = a_reg[i];
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; i++) *reinterpret_cast<u32x4*>(sb + b_dst[i]) = b_reg[i];
+    for (int i = 0; i < NINS; i++) {
+      if (i < lo || i >= hi) continue;
+      if (i < A_INS) {
+        dma16(a_src[i] + (int64_t)kt * a_step, sa + (i * NW + wave) * 1024);
+      } else {
+        const int j = i - A_INS;
+        dma16(b_src[j] + (int64_t)kt * b_step, sb + (j * NW + wave) * 1024);
+      }
+    }
   };
 
   // lane-constant parts of the LDS fragment addresses
   const int l32 = lane & 31, lhi = lane >> 5;
   // transposed-read geometry: 16-lane group g: column half = g & 1, k-group = g >> 1
   const int j16 = lane & 15, g16 = lane >> 4;
-  const int tr_krow = ((g16 >> 1) << 3) + (j16 >> 2);        // + kk*16 (+4 for second read)
-  const int tr_col = ((g16 & 1) << 4) + ((j16 & 3) << 2);     // element offset inside 32-wide tile
+  const int tr_krow = ((g16 >> 1) << 3) + (j16 >> 2);      // + kk*16 (+4 for the second read)
+  const int tr_col = ((g16 & 1) << 4) + ((j16 & 3) << 2);   // element offset inside a 32-wide tile
 
-  auto compute = [&](int stage) {
-    const unsigned char* sa = smem + stage * (A_BYTES + B_BYTES);
-    const unsigned char* sb = sa + A_BYTES;
+  auto step = [&](const unsigned char* sa, const unsigned char* sb, int kk) {
+    bf16x8 af[TM], bfr[TN];
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; kk++) {
-      bf16x8 af[TM], bfr[TN];
+    for (int i = 0; i < TM; i++) {
+      if (A_KC) {
+        const int row = wm * WM + i * 32 + l32;
+        const int ch = kk * 2 + lhi;
+        af[i] = *reinterpret_cast<const bf16x8*>(sa + row * 128 + ((ch ^ ((row >> 1) & 7)) << 4));
+      } else {
+        const int col = wm * WM + i * 32 + tr_col;
+        Pack8 p;
 #pragma unroll
-      for (int i = 0; i < TM; i++) {
-        if (A_KC) {
-          const int row = wm * WM + i * 32 + l32;
-          const int ch = kk * 2 + lhi;
-          af[i] = *reinterpret_cast<const bf16x8*>(sa + row * 128 + ((ch ^ (row & 7)) << 4));
-        } else {
-          const int col = wm * WM + i * 32 + tr_col;
-          Pack8 p;
-#pragma unroll
-          for (int h = 0; h < 2; h++) {
-            const int kr = kk * 16 + tr_krow + h * 4;
-            const int off = kr * (BM * 2) + (((col >> 3) ^ ((kr & 3) << 1)) << 4) + ((col & 7) << 1);
-            s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (s16x4 __attribute__((address_space(3)))*)(sa + off));
-            p.u[h * 2 + 0] = ((u32x2&)t)[0];
-            p.u[h * 2 + 1] = ((u32x2&)t)[1];
-          }
-          af[i] = p.v;
+        for (int h = 0; h < 2; h++) {
+          const int kr = kk * 16 + tr_krow + h * 4;
+          const int off = kr * (BM * 2) + (((col >> 3) ^ ((kr & 3) << 2)) << 4) + ((col & 7) << 1);
+          s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (s16x4 __attribute__((address_space(3)))*)(sa + off));
+          p.u[h * 2 + 0] = ((u32x2&)t)[0];
+          p.u[h * 2 + 1] = ((u32x2&)t)[1];
         }
+        af[i] = p.v;
       }
-#pragma unroll
-      for (int j = 0; j < TN; j++) {
-        if (B_KC) {
-          const int row = wn * WN + j * 32 + l32;
-          const int ch = kk * 2 + lhi;
-          bfr[j] = *reinterpret_cast<const bf16x8*>(sb + row * 128 + ((ch ^ (row & 7)) << 4));
-        } else {
-          const int col = wn * WN + j * 32 + tr_col;
-          Pack8 p;
-#pragma unroll
-          for (int h = 0; h < 2; h++) {
-            const int kr = kk * 16 + tr_krow + h * 4;
-            const int off = kr * (BN * 2) + (((col >> 3) ^ ((kr & 3) << 1)) << 4) + ((col & 7) << 1);
-            s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (s16x4 __attribute__((address_space(3)))*)(sb + off));
-            p.u[h * 2 + 0] = ((u32x2&)t)[0];
-            p.u[h * 2 + 1] = ((u32x2&)t)[1];
-          }
-          bfr[j] = p.v;
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
     }
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      if (B_KC) {
+        const int row = wn * WN + j * 32 + l32;
+        const int ch = kk * 2 + lhi;
+        bfr[j] = *reinterpret_cast<const bf16x8*>(sb + row * 128 + ((ch ^ ((row >> 1) & 7)) << 4));
+      } else {
+        const int col = wn * WN + j * 32 + tr_col;
+        Pack8 p;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const int kr = kk * 16 + tr_krow + h * 4;
+          const int off = kr * (BN * 2) + (((col >> 3) ^ ((kr & 3) << 2)) << 4) + ((col & 7) << 1);
+          s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (s16x4 __attribute__((address_space(3)))*)(sb + off));
+          p.u[h * 2 + 0] = ((u32x2&)t)[0];
+          p.u[h * 2 + 1] = ((u32x2&)t)[1];
+        }
+        bfr[j] = p.v;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
   };
 
-  gload(0);
-  lstore(0);
+  dma(0, 0, 0, NINS);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   for (int kt = 0; kt < KT; kt++) {
     const int cur = kt & 1;
-    if (kt + 1 < KT) gload(kt + 1);
-    compute(cur);
-    if (kt + 1 < KT) lstore(cur ^ 1);
+    const unsigned char* sa = smem + cur * STAGE;
+    const unsigned char* sb = sa + A_BYTES;
+    const bool more = kt + 1 < KT;
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; kk++) {
+      // the next k-tile streams into the other stage while this one is consumed; its DMA
+      // instructions are spread over the four k-steps so that no wave stalls on a full queue
+      if (more) dma(kt + 1, cur ^ 1, kk * NINS / 4, (kk + 1) * NINS / 4);
+      step(sa, sb, kk);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
 
-  // ---- epilogue: accumulator (lane -> column l32, rows 8*(r/4) + 4*lhi + r%4) ----
+  // ---- epilogue: accumulator lane -> column l32, rows 8*(r/4) + 4*lhi + r%4.  Each store
+  // instruction writes two 64-byte row segments; measured faster than 8-byte per-row stores
+  // (one lane per row), which touch 32 cache lines per instruction.
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
