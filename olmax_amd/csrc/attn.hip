@@ -59,6 +59,20 @@ __device__ __forceinline__ bf16x8 frag_tr(const unsigned char* tile, int r0, int
   return p.v;
 }
 
+// Stream ROWS rows of 128 bf16 (global row r0 + i, clamped to S-1, row stride ld) into the
+// swizzled LDS tile at lds_addr: ROWS/4 DMA instructions of 1 KB (4 rows) shared by 4 waves.
+template <int ROWS>
+__device__ __forceinline__ void dma_tile(const bf16* base, int64_t ld, int r0, int S, unsigned lds_addr, int wave, int lane) {
+#pragma unroll
+  for (int i = 0; i < ROWS / 16; i++) {
+    const int blk = i * 4 + wave;
+    const int p = blk * 64 + lane;
+    const int row = p >> 4, ph = p & 15;
+    const int gr = min(r0 + row, S - 1);
+    dma16(base + (int64_t)gr * ld + ((ph ^ swz(row)) << 3), lds_addr + blk * 1024);
+  }
+}
+
 __device__ __forceinline__ bf16x8 pack_bf16x8(const f32x16& a, int base) {
   bf16x8 r;
 #pragma unroll
@@ -108,39 +122,22 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
     for (int r = 0; r < 16; r++) o[dt][r] = 0.f;
   float m = -INFINITY, lsum = 0.f;
 
-  // tile loader: 64 rows x 16 chunks for K and V -> 4 + 4 chunks per thread
-  u32x4 kreg[4], vreg[4];
   const bf16* kbase = K + (int64_t)b * S * ldk + kh * 128;
   const bf16* vbase = V + (int64_t)b * S * ldv + kh * 128;
-  auto gload = [&](int t) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int q = i * 256 + tid;
-      const int row = q >> 4, c = q & 15;
-      const int j = min(t * 64 + row, S - 1);
-      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)j * ldk + c * 8);
-      vreg[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)j * ldv + c * 8);
-    }
-  };
-  auto lstore = [&](int stage) {
-    unsigned char* sk = smem + stage * 32768;
-    unsigned char* sv = sk + 16384;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int q = i * 256 + tid;
-      const int row = q >> 4, c = q & 15;
-      *reinterpret_cast<u32x4*>(sk + tile_off(row, c)) = kreg[i];
-      *reinterpret_cast<u32x4*>(sv + tile_off(row, c)) = vreg[i];
-    }
+  const unsigned lds0 = lds_addr_of(smem);
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
+  auto load_kv = [&](int t, int stage) {
+    dma_tile<64>(kbase, ldk, t * 64, S, lds0 + stage * 32768, wv, lane);
+    dma_tile<64>(vbase, ldv, t * 64, S, lds0 + stage * 32768 + 16384, wv, lane);
   };
   const float sc2 = scale * LOG2E;
 
-  gload(t_lo);
-  lstore(0);
+  load_kv(t_lo, 0);
+  dma_wait_all();
   __syncthreads();
   for (int t = t_lo; t <= t_hi; t++) {
     const int cur = (t - t_lo) & 1;
-    if (t < t_hi) gload(t + 1);
+    if (t < t_hi) load_kv(t + 1, cur ^ 1);
     const int j0 = t * 64;
     // skip tiles this wave cannot see at all
     const bool visible = (j0 <= iw0 + 31) && (window < 0 || j0 + 63 >= iw0 - window);
@@ -201,7 +198,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
         for (int dt = 0; dt < 4; dt++)
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(sv, u * 16, dt * 32, lane), pb[u], o[dt], 0, 0, 0);
     }
-    if (t < t_hi) lstore(cur ^ 1);
+    dma_wait_all();
     __syncthreads();
   }
   const float ltot = lsum + __shfl_xor(lsum, 32, 64);
@@ -249,7 +246,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict_
 // dQ.  Same tiling as the forward: grid = (ceil(S/128), H, B); K/V tiles stream through LDS.
 // ---------------------------------------------------------------------------------------
 template <bool CAP>
-__global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     const bf16* __restrict__ Q, const bf16* __restrict__ K, const bf16* __restrict__ V,
     const bf16* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ DELTA,
     bf16* __restrict__ dQ, int S, int H, int KH, int64_t ldq, int64_t ldk, int64_t ldv, int64_t lddo,
@@ -287,38 +284,22 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(
 #pragma unroll
     for (int r = 0; r < 16; r++) dq[dt][r] = 0.f;
 
-  u32x4 kreg[4], vreg[4];
   const bf16* kbase = K + (int64_t)b * S * ldk + kh * 128;
   const bf16* vbase = V + (int64_t)b * S * ldv + kh * 128;
-  auto gload = [&](int t) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int q = i * 256 + tid;
-      const int row = q >> 4, c = q & 15;
-      const int j = min(t * 64 + row, S - 1);
-      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)j * ldk + c * 8);
-      vreg[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)j * ldv + c * 8);
-    }
-  };
-  auto lstore = [&](int stage) {
-    unsigned char* sk = smem + stage * 32768;
-    unsigned char* sv = sk + 16384;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int q = i * 256 + tid;
-      const int row = q >> 4, c = q & 15;
-      *reinterpret_cast<u32x4*>(sk + tile_off(row, c)) = kreg[i];
-      *reinterpret_cast<u32x4*>(sv + tile_off(row, c)) = vreg[i];
-    }
+  const unsigned lds0 = lds_addr_of(smem);
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
+  auto load_kv = [&](int t, int stage) {
+    dma_tile<64>(kbase, ldk, t * 64, S, lds0 + stage * 32768, wv, lane);
+    dma_tile<64>(vbase, ldv, t * 64, S, lds0 + stage * 32768 + 16384, wv, lane);
   };
   const float sc2 = scale * LOG2E;
 
-  gload(t_lo);
-  lstore(0);
+  load_kv(t_lo, 0);
+  dma_wait_all();
   __syncthreads();
   for (int t = t_lo; t <= t_hi; t++) {
     const int cur = (t - t_lo) & 1;
-    if (t < t_hi) gload(t + 1);
+    if (t < t_hi) load_kv(t + 1, cur ^ 1);
     const int j0 = t * 64;
     const bool visible = (j0 <= iw0 + 31) && (window < 0 || j0 + 63 >= iw0 - window);
     if (visible) {
@@ -361,7 +342,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(
         for (int dt = 0; dt < 4; dt++)
           dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(sk, u * 16, dt * 32, lane), dsb[u], dq[dt], 0, 0, 0);
     }
-    if (t < t_hi) lstore(cur ^ 1);
+    dma_wait_all();
     __syncthreads();
   }
   if (qi < S) {
@@ -379,18 +360,19 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// dK/dV.  grid = (ceil(S/128), KH, B); wave w owns keys j0+32w..+31; loops over the query
-// heads of its group and over 64-row Q/dO tiles from the diagonal downwards.
-// LDS per stage: Q 16K | dO 16K | lse 256 B | delta 256 B
+// dK/dV.  grid = (ceil(S/128), KH, B); wave w owns keys j0+32w..+31 (K and V fragments stay in
+// registers); loops over the query heads of its group and over 32-row Q/dO tiles from the
+// diagonal downwards.  LDS: 2 stages of (Q 8K | dO 8K | lse 128 B | delta 128 B) + V tile 32K.
 // ---------------------------------------------------------------------------------------
 template <bool CAP>
-__global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(
+__global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
     const bf16* __restrict__ Q, const bf16* __restrict__ K, const bf16* __restrict__ V,
     const bf16* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ DELTA,
     bf16* __restrict__ dK, bf16* __restrict__ dV, int S, int H, int KH, int64_t ldq, int64_t ldk,
     int64_t ldv, int64_t lddo, int64_t lddk, int64_t lddv, float scale, int window, float cap) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  constexpr int STAGE = 32768 + 512;
+  constexpr int QT = 32;                   // query rows per iteration
+  constexpr int STAGE = 2 * QT * 256 + 256;  // Q | dO | lse, delta
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
   const int kt = blockIdx.x;
@@ -401,15 +383,13 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(
   const int kj = jw0 + l32;  // this lane's key
   const int kjc = min(kj, S - 1);
 
-  bf16x8 kf[8], vf[8];
+  // K fragments of this wave's 32 keys stay in registers; the V tile of the whole workgroup
+  // (128 keys) is parked in LDS behind the two stages and re-read as B operand every iteration
+  bf16x8 kf[8];
   {
     const bf16* kp = K + ((int64_t)b * S + kjc) * ldk + kh * 128 + lhi * 8;
-    const bf16* vp = V + ((int64_t)b * S + kjc) * ldv + kh * 128 + lhi * 8;
 #pragma unroll
-    for (int s = 0; s < 8; s++) {
-      kf[s] = *reinterpret_cast<const bf16x8*>(kp + s * 16);
-      vf[s] = *reinterpret_cast<const bf16x8*>(vp + s * 16);
-    }
+    for (int s = 0; s < 8; s++) kf[s] = *reinterpret_cast<const bf16x8*>(kp + s * 16);
   }
   f32x16 dk[4], dv[4];
 #pragma unroll
@@ -418,112 +398,97 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(
     for (int r = 0; r < 16; r++) { dk[dt][r] = 0.f; dv[dt][r] = 0.f; }
 
   const int i_hi = window >= 0 ? min(S - 1, j0 + 127 + window) : S - 1;
-  const int t_lo = j0 >> 6;
-  const int t_hi = i_hi >> 6;  // inclusive, 64-row query tiles
+  const int t_lo = j0 / QT;
+  const int t_hi = i_hi / QT;  // inclusive
   const int ntile = t_hi - t_lo + 1;
   const int total = ntile * rep;  // flattened (head, tile) iteration space
   const float sc2 = scale * LOG2E;
+  const unsigned lds0 = lds_addr_of(smem);
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
 
-  u32x4 qreg[4], oreg[4];
   float sreg = 0.f;
-  auto gload = [&](int it) {
+  auto load_tile = [&](int it, int stage) {
     const int hq = kh * rep + it / ntile;
     const int t = t_lo + it % ntile;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int q = i * 256 + tid;
-      const int row = q >> 4, c = q & 15;
-      const int ii = min(t * 64 + row, S - 1);
-      qreg[i] = *reinterpret_cast<const u32x4*>(Q + ((int64_t)b * S + ii) * ldq + hq * 128 + c * 8);
-      oreg[i] = *reinterpret_cast<const u32x4*>(dO + ((int64_t)b * S + ii) * lddo + hq * 128 + c * 8);
-    }
-    if (tid < 128) {
-      const int ii = min(t * 64 + (tid & 63), S - 1);
-      const float* src = tid < 64 ? LSE : DELTA;
+    dma_tile<QT>(Q + (int64_t)b * S * ldq + hq * 128, ldq, t * QT, S, lds0 + stage * STAGE, wv, lane);
+    dma_tile<QT>(dO + (int64_t)b * S * lddo + hq * 128, lddo, t * QT, S, lds0 + stage * STAGE + QT * 256, wv, lane);
+    if (tid < 2 * QT) {
+      const int ii = min(t * QT + (tid & (QT - 1)), S - 1);
+      const float* src = tid < QT ? LSE : DELTA;
       sreg = src[((int64_t)b * H + hq) * S + ii];
-      if (tid < 64) sreg *= LOG2E;
+      if (tid < QT) sreg *= LOG2E;
     }
   };
-  auto lstore = [&](int stage) {
-    unsigned char* sq = smem + stage * STAGE;
-    unsigned char* so = sq + 16384;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int q = i * 256 + tid;
-      const int row = q >> 4, c = q & 15;
-      *reinterpret_cast<u32x4*>(sq + tile_off(row, c)) = qreg[i];
-      *reinterpret_cast<u32x4*>(so + tile_off(row, c)) = oreg[i];
-    }
-    if (tid < 128) reinterpret_cast<float*>(sq + 32768)[tid] = sreg;
+  auto store_stats = [&](int stage) {
+    if (tid < 2 * QT) reinterpret_cast<float*>(smem + stage * STAGE + 2 * QT * 256)[tid] = sreg;
   };
 
-  gload(0);
-  lstore(0);
+  const unsigned char* svt = smem + 2 * STAGE;  // [128 keys][128] V tile
+  dma_tile<128>(V + (int64_t)b * S * ldv + kh * 128, ldv, j0, S, lds0 + 2 * STAGE, wv, lane);
+  load_tile(0, 0);
+  store_stats(0);
+  dma_wait_all();
   __syncthreads();
   for (int it = 0; it < total; it++) {
     const int cur = it & 1;
-    if (it + 1 < total) gload(it + 1);
+    if (it + 1 < total) load_tile(it + 1, cur ^ 1);
     const int t = t_lo + it % ntile;
-    const int ib = t * 64;  // first query of the tile
-    // this wave sees the tile iff some i in [ib, ib+63] has j <= i <= j + window for its keys
-    const bool visible = (ib + 63 >= jw0) && (window < 0 || ib <= jw0 + 31 + window);
+    const int ib = t * QT;  // first query of the tile
+    // this wave sees the tile iff some i in [ib, ib+QT) has j <= i <= j + window for its keys
+    const bool visible = (ib + QT - 1 >= jw0) && (window < 0 || ib <= jw0 + 31 + window);
     if (visible) {
       const unsigned char* sq = smem + cur * STAGE;
-      const unsigned char* so = sq + 16384;
-      const float* slse = reinterpret_cast<const float*>(sq + 32768);
-      const float* sdel = slse + 64;
-      f32x16 sa[2], dpa[2];
+      const unsigned char* so = sq + QT * 256;
+      const float* slse = reinterpret_cast<const float*>(sq + 2 * QT * 256);
+      const float* sdel = slse + QT;
+      f32x16 sa, dpa;
 #pragma unroll
-      for (int itl = 0; itl < 2; itl++) {
+      for (int r = 0; r < 16; r++) { sa[r] = 0.f; dpa[r] = 0.f; }
 #pragma unroll
-        for (int r = 0; r < 16; r++) { sa[itl][r] = 0.f; dpa[itl][r] = 0.f; }
-#pragma unroll
-        for (int s = 0; s < 8; s++) {
-          sa[itl] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sq, itl * 32 + l32, s, lhi), kf[s], sa[itl], 0, 0, 0);
-          dpa[itl] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(so, itl * 32 + l32, s, lhi), vf[s], dpa[itl], 0, 0, 0);
-        }
+      for (int s = 0; s < 8; s++) {
+        sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sq, l32, s, lhi), kf[s], sa, 0, 0, 0);
+        dpa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(so, l32, s, lhi), frag_kc(svt, wave * 32 + l32, s, lhi), dpa, 0, 0, 0);
       }
-      // accumulator rows are queries i = ib + 32*itl + 8*(r/4) + 4*lhi + r%4; column = key kj
+      // accumulator rows are queries i = ib + 8*(r/4) + 4*lhi + r%4; column = key kj
 #pragma unroll
-      for (int itl = 0; itl < 2; itl++)
+      for (int g = 0; g < 4; g++) {
+        const int il = g * 8 + lhi * 4;
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(slse + il);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(sdel + il);
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const int il = itl * 32 + g * 8 + lhi * 4;
-          const f32x4 l4 = *reinterpret_cast<const f32x4*>(slse + il);
-          const f32x4 d4 = *reinterpret_cast<const f32x4*>(sdel + il);
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const int r = g * 4 + e;
-            const int i = ib + il + e;
-            float s = sa[itl][r], chain = 1.f;
-            if (CAP) {
-              const float th = fast_tanh(s * scale / cap);
-              s = cap * th * LOG2E;
-              chain = 1.f - th * th;
-            } else {
-              s = s * sc2;
-            }
-            const bool ok = (kj <= i) && (i < S) && (window < 0 || kj >= i - window);
-            const float p = ok ? fexp2(s - l4[e]) : 0.f;
-            sa[itl][r] = p;
-            dpa[itl][r] = p * (dpa[itl][r] - d4[e]) * chain;
+        for (int e = 0; e < 4; e++) {
+          const int r = g * 4 + e;
+          const int i = ib + il + e;
+          float s = sa[r], chain = 1.f;
+          if (CAP) {
+            const float th = fast_tanh(s * scale / cap);
+            s = cap * th * LOG2E;
+            chain = 1.f - th * th;
+          } else {
+            s = s * sc2;
           }
+          const bool ok = (kj <= i) && (i < S) && (window < 0 || kj >= i - window);
+          const float p = ok ? fexp2(s - l4[e]) : 0.f;
+          sa[r] = p;
+          dpa[r] = p * (dpa[r] - d4[e]) * chain;
         }
-      bf16x8 pb[4], dsb[4];
+      }
+      bf16x8 pb[2], dsb[2];
 #pragma unroll
-      for (int u = 0; u < 4; u++) {
-        pb[u] = pack_bf16x8(sa[u >> 1], (u & 1) * 8);
-        dsb[u] = pack_bf16x8(dpa[u >> 1], (u & 1) * 8);
+      for (int u = 0; u < 2; u++) {
+        pb[u] = pack_bf16x8(sa, u * 8);
+        dsb[u] = pack_bf16x8(dpa, u * 8);
       }
 #pragma unroll
-      for (int u = 0; u < 4; u++)
+      for (int u = 0; u < 2; u++)
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) {
           dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(so, u * 16, dt * 32, lane), pb[u], dv[dt], 0, 0, 0);
           dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(sq, u * 16, dt * 32, lane), dsb[u], dk[dt], 0, 0, 0);
         }
     }
-    if (it + 1 < total) lstore(cur ^ 1);
+    if (it + 1 < total) store_stats(cur ^ 1);
+    dma_wait_all();
     __syncthreads();
   }
   if (kj < S) {
@@ -712,7 +677,7 @@ extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void*
     const int64_t units = (int64_t)B * S * H;
     hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((units + 15) / 16)), dim3(256), 0, stream, op, gop, delta, B, S, H, ldo, lddo);
     dim3 gkv((S + 127) / 128, KH, B), gq((S + 127) / 128, H, B);
-    constexpr int SM_KV = 2 * (32768 + 512);
+    constexpr int SM_KV = 2 * (2 * 32 * 256 + 256) + 128 * 256;
     static bool set = false;
     if (!set) {
       (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);

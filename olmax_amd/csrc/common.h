@@ -55,6 +55,18 @@ union Pack4 {
   bf16 e[4];
 };
 
+// 16 B per lane straight from global memory into LDS at (lds_addr + lane*16); lds_addr is
+// wave-uniform (it travels in M0).  Issued as inline asm so that the compiler does not
+// serialise later LDS reads behind it; the issuer waits for completion explicitly
+// (s_waitcnt vmcnt) before the barrier that publishes the data.
+__device__ __forceinline__ void dma16(const void* g, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(g) : "m0", "memory");
+}
+__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ unsigned lds_addr_of(const void* p) {
+  return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)p;
+}
+
 // Wave64 all-reduce (sum) by xor shuffles.
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

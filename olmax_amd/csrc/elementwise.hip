@@ -152,36 +152,53 @@ __global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ p, const
                                                     const float* __restrict__ gscale_dev) {
   if (gscale_dev) gscale *= *gscale_dev;
   const int64_t n4 = n / 4;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
-    f32x4 pv = reinterpret_cast<const f32x4*>(p)[i];
-    f32x4 mv = reinterpret_cast<const f32x4*>(m)[i];
-    f32x4 vv = reinterpret_cast<const f32x4*>(v)[i];
-    float g[4];
-    if (G_BF16) {
-      Pack4 gp;
-      gp.u = reinterpret_cast<const u32x2*>(gv)[i];
+  const float ibc1 = 1.f / bc1, ibc2 = 1.f / bc2, omb1 = 1.f - b1, omb2 = 1.f - b2;
+  // every element is touched exactly once: streaming (non-temporal) accesses keep the 28 B/param
+  // out of the way of the L2; two 16-byte groups per lane per iteration for more bytes in flight
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i0 = (int64_t)blockIdx.x * 256 + threadIdx.x; i0 < n4; i0 += 2 * stride) {
+    f32x4 pv[2], mv[2], vv[2];
+    float g[2][4];
+    bool live[2];
 #pragma unroll
-      for (int e = 0; e < 4; e++) g[e] = bf2f(gp.e[e]);
-    } else {
-      f32x4 gf = reinterpret_cast<const f32x4*>(gv)[i];
+    for (int u = 0; u < 2; u++) {
+      const int64_t i = i0 + u * stride;
+      live[u] = i < n4;
+      if (!live[u]) continue;
+      pv[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p) + i);
+      mv[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(m) + i);
+      vv[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(v) + i);
+      if (G_BF16) {
+        Pack4 gp;
+        gp.u = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(gv) + i);
 #pragma unroll
-      for (int e = 0; e < 4; e++) g[e] = gf[e];
+        for (int e = 0; e < 4; e++) g[u][e] = bf2f(gp.e[e]);
+      } else {
+        f32x4 gf = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(gv) + i);
+#pragma unroll
+        for (int e = 0; e < 4; e++) g[u][e] = gf[e];
+      }
     }
-    Pack4 sh;
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-      const float ge = g[e] * gscale;
-      mv[e] = b1 * mv[e] + (1.f - b1) * ge;
-      vv[e] = b2 * vv[e] + (1.f - b2) * ge * ge;
-      const float mh = mv[e] / bc1;
-      const float vh = vv[e] / bc2;
-      pv[e] = pv[e] - lr * (mh / (sqrtf(vh) + eps) + wd * pv[e]);
-      sh.e[e] = f2bf(pv[e]);
+    for (int u = 0; u < 2; u++) {
+      if (!live[u]) continue;
+      const int64_t i = i0 + u * stride;
+      Pack4 sh;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const float ge = g[u][e] * gscale;
+        mv[u][e] = b1 * mv[u][e] + omb1 * ge;
+        vv[u][e] = b2 * vv[u][e] + omb2 * ge * ge;
+        const float mh = mv[u][e] * ibc1;
+        const float vh = vv[u][e] * ibc2;
+        pv[u][e] = pv[u][e] - lr * (mh / (sqrtf(vh) + eps) + wd * pv[u][e]);
+        sh.e[e] = f2bf(pv[u][e]);
+      }
+      __builtin_nontemporal_store(pv[u], reinterpret_cast<f32x4*>(p) + i);
+      __builtin_nontemporal_store(mv[u], reinterpret_cast<f32x4*>(m) + i);
+      __builtin_nontemporal_store(vv[u], reinterpret_cast<f32x4*>(v) + i);
+      if (shadow) __builtin_nontemporal_store(sh.u, reinterpret_cast<u32x2*>(shadow) + i);
     }
-    reinterpret_cast<f32x4*>(p)[i] = pv;
-    reinterpret_cast<f32x4*>(m)[i] = mv;
-    reinterpret_cast<f32x4*>(v)[i] = vv;
-    if (shadow) reinterpret_cast<u32x2*>(shadow)[i] = sh.u;
   }
   // tail (n % 4) handled by the first threads of block 0
   if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
@@ -329,7 +346,7 @@ extern "C" int32_t olmax_adamw_dscale(hipStream_t stream, float* p, const void* 
               OLMAX_ERR_ALIGN, "olmax_adamw: buffers must be 16-byte aligned (bf16 buffers 8-byte)");
   const float bc1 = (float)(1.0 - pow((double)b1, (double)step));
   const float bc2 = (float)(1.0 - pow((double)b2, (double)step));
-  const int grid = grid_1d((n + 3) / 4, 16384);
+  const int grid = grid_1d((n + 7) / 8, 8192);
   if (grad_is_bf16)
     hipLaunchKernelGGL(adamw_kernel<true>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale, grad_scale_dev);
   else

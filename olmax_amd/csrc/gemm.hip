@@ -49,14 +49,6 @@ bool g_prof_on = false;
 std::vector<ProfRec> g_prof;
 std::mutex g_prof_mu;
 
-// 16 B per lane straight from global memory into LDS at (lds_addr + lane*16); lds_addr is
-// wave-uniform (it travels in M0).  Issued as inline asm so that the compiler does not
-// serialise later LDS reads behind it; completion is awaited explicitly (vmcnt) before the
-// barrier that publishes the tile.
-__device__ __forceinline__ void dma16(const void* g, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(g) : "m0", "memory");
-}
-
 template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
     const bf16* __restrict__ A, const bf16* __restrict__ B, void* __restrict__ Cv,
@@ -136,7 +128,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
   const int KT = K / BK;
-  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  const unsigned lds_base = lds_addr_of(smem);
   // issue DMA instructions [lo, hi) of the combined A+B list of k-tile kt into `stage`
   auto dma = [&](int kt, int stage, int lo, int hi) {
     const unsigned sa = lds_base + stage * STAGE;
@@ -212,7 +204,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
   };
 
   dma(0, 0, 0, NINS);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  dma_wait_all();
   __syncthreads();
   for (int kt = 0; kt < KT; kt++) {
     const int cur = kt & 1;
@@ -226,7 +218,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
       if (more) dma(kt + 1, cur ^ 1, kk * NINS / 4, (kk + 1) * NINS / 4);
       step(sa, sb, kk);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    dma_wait_all();
     __syncthreads();
   }
 

@@ -123,8 +123,11 @@ int lin_dw(hipStream_t s, const bf16* dy, int64_t lddy, const bf16* x, int64_t l
   return olmax_gemm_bf16(s, dy, x, dW, nullptr, out, in, (int)T, lddy, ldx, in, 0, 1, 1, out_f32);
 }
 
+// need_y == false (recompute before the backward): the block output itself is not an input of
+// the backward pass, so the GEMM / norm that only produces it is skipped.
 int block_forward(hipStream_t s, const olmax_model_config* c, const olmax_block_weights* w, int window,
-                  const float* cos_t, const float* sin_t, const bf16* x, bf16* y, const Acts& a) {
+                  const float* cos_t, const float* sin_t, const bf16* x, bf16* y, const Acts& a,
+                  bool need_y = true) {
   const Dims m = dims_of(c);
   const int lt = c->layer_type;
   const float eps = c->eps;
@@ -164,10 +167,10 @@ int block_forward(hipStream_t s, const olmax_model_config* c, const olmax_block_
   RC(lin_fwd(s, mlp_in, m.d, w->wgu, m.d, 2 * m.F, a.gu, 2 * m.F, nullptr, 0, m.T));
   RC(olmax_glu_fwd(s, a.gu, a.gu + m.F, a.act, m.T, m.F, 2 * m.F, 2 * m.F, m.F, c->act));
   if (lt == 0) {
-    RC(lin_fwd(s, a.act, m.F, w->wdown, m.F, m.d, y, m.d, a.h, m.d, m.T));
+    if (need_y) RC(lin_fwd(s, a.act, m.F, w->wdown, m.F, m.d, y, m.d, a.h, m.d, m.T));
   } else {
     RC(lin_fwd(s, a.act, m.F, w->wdown, m.F, m.d, a.m_out, m.d, nullptr, 0, m.T));
-    RC(olmax_rmsnorm_fwd_res(s, a.m_out, w->mlp_norm, a.h, y, m.T, m.d, m.d, m.d, m.d, eps));
+    if (need_y) RC(olmax_rmsnorm_fwd_res(s, a.m_out, w->mlp_norm, a.h, y, m.T, m.d, m.d, m.d, m.d, eps));
   }
   return OLMAX_OK;
 }
@@ -427,8 +430,8 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
     Acts acts = carve_acts(c, aa);
     const bf16* xin = w.xs + (int64_t)l * Td;
     if (!keep) {
-      // full-block recompute; the block output itself is not needed again -> scratch into dnext
-      RC(block_forward(s, c, &bw, windows[l], cos_tables[l], sin_tables[l], xin, dnext, acts));
+      // full-block recompute of everything the backward reads
+      RC(block_forward(s, c, &bw, windows[l], cos_tables[l], sin_tables[l], xin, dnext, acts, false));
     }
     RC(block_backward(s, c, &bw, &bg, windows[l], cos_tables[l], sin_tables[l], xin, dcur, dnext, acts, w.tmp));
     bf16* t = dcur;

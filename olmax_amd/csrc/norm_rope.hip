@@ -459,11 +459,11 @@ extern "C" int32_t olmax_rmsnorm_bwd(hipStream_t stream, const void* x, const vo
   bf16* dxp = (bf16*)dx;
   const size_t smem = dw ? (size_t)d * 4 : 0;
   if (vec && d % 8 == 0 && d <= 256) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<16, 2>), dim3(grid_for(rows, 16, 2048)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<16, 2>), dim3(grid_for(rows, 16, 512)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   } else if (vec && d % 8 == 0 && d <= 4096) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 8>), dim3(grid_for(rows, 4, 2048)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 8>), dim3(grid_for(rows, 4, 512)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   } else if (vec && d % 8 == 0 && d <= 8192) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 16>), dim3(grid_for(rows, 4, 2048)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 16>), dim3(grid_for(rows, 4, 512)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   } else {
     hipLaunchKernelGGL(rmsnorm_bwd_generic, dim3(grid_for(rows, 1, 1 << 16)), dim3(256), 0, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   }
