@@ -37,6 +37,43 @@ __device__ __forceinline__ int swz(int row) { return ((row & 3) << 2) | ((row >>
 // byte offset of 16B chunk `c` (0..15) of row `row` in a [rows][128] bf16 tile
 __device__ __forceinline__ int tile_off(int row, int c) { return row * 256 + ((c ^ swz(row)) << 4); }
 
+// Per-lane byte offsets of the operand fragments inside a [rows][128] tile.  The swizzle only
+// looks at row bits 0-3, so stepping rows by 16 or 32 is a plain immediate offset and the
+// eight (k-contiguous) plus eight (transposed) lane-dependent offsets are loop invariant.
+struct FragAddr {
+  int kc[8];     // row (lane % 32), k-step s
+  int tr[4][2];  // column tile dt, half h of the transposed read
+  __device__ __forceinline__ void init(int lane) {
+    const int l32 = lane & 31, lhi = lane >> 5;
+#pragma unroll
+    for (int s = 0; s < 8; s++) kc[s] = l32 * 256 + (((2 * s + lhi) ^ swz(l32)) << 4);
+    const int j16 = lane & 15, g16 = lane >> 4;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int col = dt * 32 + ((g16 & 1) << 4) + ((j16 & 3) << 2);
+        const int row = ((g16 >> 1) << 2) + (h << 3) + (j16 >> 2);
+        tr[dt][h] = row * 256 + (((col >> 3) ^ swz(row)) << 4) + ((col & 7) << 1);
+      }
+  }
+  // k-contiguous fragment: rows row0 + lane%32 (row0 multiple of 16), k-step s
+  __device__ __forceinline__ bf16x8 load_kc(const unsigned char* tile, int row0, int s) const {
+    return *reinterpret_cast<const bf16x8*>(tile + kc[s] + row0 * 256);
+  }
+  // transposed fragment: MFMA rows = storage columns dt*32 + lane%32, k = storage rows r0 + {..}
+  __device__ __forceinline__ bf16x8 load_tr(const unsigned char* tile, int r0, int dt) const {
+    Pack8 p;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(tile + tr[dt][h] + r0 * 256));
+      p.u[h * 2 + 0] = ((u32x2&)t)[0];
+      p.u[h * 2 + 1] = ((u32x2&)t)[1];
+    }
+    return p.v;
+  }
+};
+
 // A/B operand fragment with the k index contiguous in storage: row `row`, k-step s (16 wide)
 __device__ __forceinline__ bf16x8 frag_kc(const unsigned char* tile, int row, int s, int lhi) {
   return *reinterpret_cast<const bf16x8*>(tile + tile_off(row, 2 * s + lhi));
@@ -131,6 +168,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
     dma_tile<64>(vbase, ldv, t * 64, S, lds0 + stage * 32768 + 16384, wv, lane);
   };
   const float sc2 = scale * LOG2E;
+  FragAddr fa;
+  fa.init(lane);
 
   load_kv(t_lo, 0);
   dma_wait_all();
@@ -146,49 +185,65 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
       const unsigned char* sv = sk + 16384;
       f32x16 st[2];
 #pragma unroll
-      for (int jt = 0; jt < 2; jt++) {
+      for (int jt = 0; jt < 2; jt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) st[jt][r] = 0.f;
 #pragma unroll
-        for (int s = 0; s < 8; s++)
-          st[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sk, jt * 32 + l32, s, lhi), qf[s], st[jt], 0, 0, 0);
+      for (int s = 0; s < 8; s++)
+#pragma unroll
+        for (int jt = 0; jt < 2; jt++)
+          st[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(sk, jt * 32, s), qf[s], st[jt], 0, 0, 0);
+      // scores in log2 units
+      if (CAP) {
+#pragma unroll
+        for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) st[jt][r] = cap * fast_tanh(st[jt][r] * scale / cap) * LOG2E;
       }
       const bool need_mask = (j0 + 63 > iw0) || (window >= 0 && j0 < iw0 + 31 - window);
+      if (need_mask) {
+#pragma unroll
+        for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int j = j0 + jt * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
+            const bool ok = (j <= qi) && (window < 0 || j >= qi - window);
+            st[jt][r] = ok ? st[jt][r] : -INFINITY;
+          }
+      }
       float mt = -INFINITY;
 #pragma unroll
       for (int jt = 0; jt < 2; jt++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          float s = st[jt][r];
-          if (CAP) s = cap * fast_tanh(s * scale / cap) * LOG2E;
-          else s = s * sc2;
-          if (need_mask) {
-            const int j = j0 + jt * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
-            const bool ok = (j <= qi) && (window < 0 || j >= qi - window);
-            s = ok ? s : -INFINITY;
-          }
-          st[jt][r] = s;
-          mt = fmaxf(mt, s);
-        }
+        for (int r = 0; r < 16; r++) mt = fmaxf(mt, st[jt][r]);
+      if (!CAP) mt *= sc2;  // sc2 > 0: the max commutes with the scaling
       mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-      const float m_new = fmaxf(m, mt);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fexp2(m - m_use);  // m = -inf -> 0
+      // Lazy rescaling: the running reference m only moves when some row's maximum grew by more
+      // than 2^8; until then exp2(s - m) <= 256 stays well inside fp32/bf16 range and the
+      // 64-register rescale of O is skipped (wave-uniform decision).
+      const bool grow = mt > m + 8.f;
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+        const float m_new = fmaxf(m, mt);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fexp2(m - m_use);  // m = -inf -> 0
+        lsum *= alpha;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+      }
+      const float m_use = (m == -INFINITY) ? 0.f : m;
       float ps = 0.f;
 #pragma unroll
       for (int jt = 0; jt < 2; jt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const float p = fexp2(st[jt][r] - m_use);
+          const float p = CAP ? fexp2(st[jt][r] - m_use) : fexp2(__builtin_fmaf(st[jt][r], sc2, -m_use));
           st[jt][r] = p;
           ps += p;
         }
-      lsum = lsum * alpha + ps;
-      m = m_new;
-#pragma unroll
-      for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+      lsum += ps;
       bf16x8 pb[4];
 #pragma unroll
       for (int u = 0; u < 4; u++) pb[u] = pack_bf16x8(st[u >> 1], (u & 1) * 8);
@@ -196,7 +251,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
       for (int u = 0; u < 4; u++)
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(sv, u * 16, dt * 32, lane), pb[u], o[dt], 0, 0, 0);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_tr(sv, u * 16, dt), pb[u], o[dt], 0, 0, 0);
     }
     dma_wait_all();
     __syncthreads();
@@ -294,6 +349,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
   };
   const float sc2 = scale * LOG2E;
 
+  FragAddr fa;
+  fa.init(lane);
+
   load_kv(t_lo, 0);
   dma_wait_all();
   __syncthreads();
@@ -305,6 +363,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     if (visible) {
       const unsigned char* sk = smem + cur * 32768;
       const unsigned char* sv = sk + 16384;
+      const bool need_mask = (j0 + 63 > iw0) || (window >= 0 && j0 < iw0 + 31 - window);
       f32x16 st[2], dpt[2];
 #pragma unroll
       for (int jt = 0; jt < 2; jt++) {
@@ -312,25 +371,27 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
         for (int r = 0; r < 16; r++) { st[jt][r] = 0.f; dpt[jt][r] = 0.f; }
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-          st[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sk, jt * 32 + l32, s, lhi), qf[s], st[jt], 0, 0, 0);
-          dpt[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sv, jt * 32 + l32, s, lhi), dof[s], dpt[jt], 0, 0, 0);
+          st[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(sk, jt * 32, s), qf[s], st[jt], 0, 0, 0);
+          dpt[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(sv, jt * 32, s), dof[s], dpt[jt], 0, 0, 0);
         }
       }
 #pragma unroll
       for (int jt = 0; jt < 2; jt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          float s = st[jt][r], chain = 1.f;
+          float s = st[jt][r], chain = 1.f, p;
           if (CAP) {
             const float th = fast_tanh(s * scale / cap);
-            s = cap * th * LOG2E;
+            p = fexp2(cap * th * LOG2E - lse2);
             chain = 1.f - th * th;
           } else {
-            s = s * sc2;
+            p = fexp2(__builtin_fmaf(s, sc2, -lse2));
           }
-          const int j = j0 + jt * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
-          const bool ok = (j <= qi) && (window < 0 || j >= qi - window);
-          const float p = ok ? fexp2(s - lse2) : 0.f;
+          if (need_mask) {
+            const int j = j0 + jt * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
+            const bool ok = (j <= qi) && (window < 0 || j >= qi - window);
+            p = ok ? p : 0.f;
+          }
           st[jt][r] = p * (dpt[jt][r] - dlt) * chain;
         }
       bf16x8 dsb[4];
@@ -340,7 +401,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
       for (int u = 0; u < 4; u++)
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
-          dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(sk, u * 16, dt * 32, lane), dsb[u], dq[dt], 0, 0, 0);
+          dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_tr(sk, u * 16, dt), dsb[u], dq[dt], 0, 0, 0);
     }
     dma_wait_all();
     __syncthreads();
@@ -423,6 +484,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
     if (tid < 2 * QT) reinterpret_cast<float*>(smem + stage * STAGE + 2 * QT * 256)[tid] = sreg;
   };
 
+  FragAddr fa;
+  fa.init(lane);
   const unsigned char* svt = smem + 2 * STAGE;  // [128 keys][128] V tile
   dma_tile<128>(V + (int64_t)b * S * ldv + kh * 128, ldv, j0, S, lds0 + 2 * STAGE, wv, lane);
   load_tile(0, 0);
@@ -441,13 +504,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
       const unsigned char* so = sq + QT * 256;
       const float* slse = reinterpret_cast<const float*>(sq + 2 * QT * 256);
       const float* sdel = slse + QT;
+      // every (query, key) pair of the tile is visible unless the tile touches the diagonal, the
+      // window edge or the end of the sequence
+      const bool need_mask = (ib < jw0 + 31) || (ib + QT > S) || (window >= 0 && ib + QT - 1 > jw0 + window);
       f32x16 sa, dpa;
 #pragma unroll
       for (int r = 0; r < 16; r++) { sa[r] = 0.f; dpa[r] = 0.f; }
 #pragma unroll
       for (int s = 0; s < 8; s++) {
-        sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(sq, l32, s, lhi), kf[s], sa, 0, 0, 0);
-        dpa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(so, l32, s, lhi), frag_kc(svt, wave * 32 + l32, s, lhi), dpa, 0, 0, 0);
+        sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(sq, 0, s), kf[s], sa, 0, 0, 0);
+        dpa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(so, 0, s), fa.load_kc(svt, wave * 32, s), dpa, 0, 0, 0);
       }
       // accumulator rows are queries i = ib + 8*(r/4) + 4*lhi + r%4; column = key kj
 #pragma unroll
@@ -459,16 +525,18 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
         for (int e = 0; e < 4; e++) {
           const int r = g * 4 + e;
           const int i = ib + il + e;
-          float s = sa[r], chain = 1.f;
+          float s = sa[r], chain = 1.f, p;
           if (CAP) {
             const float th = fast_tanh(s * scale / cap);
-            s = cap * th * LOG2E;
+            p = fexp2(cap * th * LOG2E - l4[e]);
             chain = 1.f - th * th;
           } else {
-            s = s * sc2;
+            p = fexp2(__builtin_fmaf(s, sc2, -l4[e]));
           }
-          const bool ok = (kj <= i) && (i < S) && (window < 0 || kj >= i - window);
-          const float p = ok ? fexp2(s - l4[e]) : 0.f;
+          if (need_mask) {
+            const bool ok = (kj <= i) && (i < S) && (window < 0 || kj >= i - window);
+            p = ok ? p : 0.f;
+          }
           sa[r] = p;
           dpa[r] = p * (dpa[r] - d4[e]) * chain;
         }
@@ -483,8 +551,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
       for (int u = 0; u < 2; u++)
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) {
-          dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(so, u * 16, dt * 32, lane), pb[u], dv[dt], 0, 0, 0);
-          dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(sq, u * 16, dt * 32, lane), dsb[u], dk[dt], 0, 0, 0);
+          dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_tr(so, u * 16, dt), pb[u], dv[dt], 0, 0, 0);
+          dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_tr(sq, u * 16, dt), dsb[u], dk[dt], 0, 0, 0);
         }
     }
     if (it + 1 < total) store_stats(cur ^ 1);
