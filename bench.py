@@ -63,6 +63,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-checkpoint", action="store_true", help="keep activations instead of full-block recompute")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-overlap", action="store_true", help="run AdamW after the backward pass instead of overlapping it on a second stream")
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline metric)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -86,7 +87,7 @@ def main():
     optim = AdamWConfig(lr=WarmupCosineDecaySchedule(warmup_steps=20, decay_steps=80, peak_value=1e-4,
                                                      init_value=1e-6, end_value=1e-6),
                         no_decay_modules=["embedding.weight"])
-    trainer = Trainer(model, optim)
+    trainer = Trainer(model, optim, overlap_optimizer=not args.no_overlap)
     T = B * S
     nb = 4
     gen = torch.Generator().manual_seed(0)
@@ -147,7 +148,7 @@ def main():
                                "SwiGLU 11008, vocab 100352 untied, seq 4096, micro-batch 2, bf16 compute, fp32 master + "
                                "AdamW, " + ("activations kept (no recompute)" if args.no_checkpoint else "full-block activation checkpointing"),
                    "layers": cfg.num_layers, "global_batch": B, "seq_len": S, "params": model.num_params,
-                   "activation_checkpointing": not args.no_checkpoint},
+                   "activation_checkpointing": not args.no_checkpoint, "optimizer_overlap": not args.no_overlap},
         "roofline": roofline,
         "gemm_kernels": per[:6],
     }

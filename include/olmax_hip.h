@@ -229,6 +229,18 @@ int32_t olmax_model_adamw(olmax_stream_t stream, const olmax_model_config* cfg, 
                           const float* grad_f32, int64_t step, float lr, float b1, float b2, float eps,
                           float wd, int32_t decay_embedding, float max_grad_norm, float* norm_scratch);
 
+/* process_microbatch, src/olmax/train/trainer.py:759-777: loss + gradients + AdamW in one call.
+ * opt_stream (optional, default priority, != stream): when given and clipping is off, each
+ * layer's AdamW runs there concurrently with the backward pass of the layers below it, and
+ * `stream` waits for it at the end.  Creates one HIP event per host thread on first use. */
+int32_t olmax_model_train_step(olmax_stream_t stream, olmax_stream_t opt_stream, const olmax_model_config* cfg,
+                               const int32_t* windows, const float* const* cos_tables,
+                               const float* const* sin_tables, float* master, float* m, float* v,
+                               void* params_bf16, const int32_t* ids, const int32_t* labels, float* loss,
+                               void* grad_bf16, float* grad_f32, void* workspace, int64_t workspace_bytes,
+                               int64_t step, float lr, float b1, float b2, float eps, float wd,
+                               int32_t decay_embedding, float max_grad_norm, float* norm_scratch);
+
 /* Single transformer block in isolation (any of the three orderings). */
 typedef struct {
   const void *wqkv, *wo, *wgu, *wdown;          /* bf16: [(H+2K)D, d], [d, HD], [2F, d], [d, F] */

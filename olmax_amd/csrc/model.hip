@@ -366,9 +366,18 @@ void fill_grads(bf16* G, float* Gf, const LayerOff& o, olmax_block_grads& g) {
   g.k_norm = o.f_k_norm >= 0 ? Gf + o.f_k_norm : nullptr;
 }
 
+// Called from model_run when every gradient of a group of leaves is final:
+// layer >= 0: that layer's leaves; -1: final norm and (untied) LM head; -2: embedding.
+struct GradReady {
+  int (*fn)(void* ctx, int layer) = nullptr;
+  void* ctx = nullptr;
+  int operator()(int layer) const { return fn ? fn(ctx, layer) : OLMAX_OK; }
+};
+
 int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows, const float* const* cos_tables,
               const float* const* sin_tables, const void* params_bf16, const int32_t* ids, const int32_t* labels,
-              float* loss, void* grad_bf16, float* grad_f32, void* workspace, int64_t workspace_bytes, bool bwd) {
+              float* loss, void* grad_bf16, float* grad_f32, void* workspace, int64_t workspace_bytes, bool bwd,
+              GradReady ready = GradReady()) {
   RC(check_cfg(c));
   OLMAX_CHECK(params_bf16 && ids && labels && loss && workspace, OLMAX_ERR_ARG, "olmax_model: null pointer");
   OLMAX_CHECK(!bwd || (grad_bf16 && grad_f32), OLMAX_ERR_ARG, "olmax_model: gradient buffers are null");
@@ -417,6 +426,7 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
   }
   RC(olmax_rmsnorm_bwd(s, xl, P + L.final_norm, w.da, nullptr, w.db, grad_f32 + L.f_final_norm, m.T, m.d, m.d, m.d, 0,
                        m.d, c->eps));
+  RC(ready(-1));
   bf16* dcur = w.db;
   bf16* dnext = w.da;
   for (int l = nl - 1; l >= 0; l--) {
@@ -434,12 +444,77 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
       RC(block_forward(s, c, &bw, windows[l], cos_tables[l], sin_tables[l], xin, dnext, acts, false));
     }
     RC(block_backward(s, c, &bw, &bg, windows[l], cos_tables[l], sin_tables[l], xin, dcur, dnext, acts, w.tmp));
+    RC(ready(l));
     bf16* t = dcur;
     dcur = dnext;
     dnext = t;
   }
   RC(olmax_embed_bwd(s, ids, dcur, grad_f32 + L.f_embedding, m.T, m.d, c->vocab));
+  RC(ready(-2));
   return OLMAX_OK;
+}
+
+// AdamW over the leaves [begin, end) of a layout; runs of adjacent bf16-gradient leaves with
+// the same decay become single launches.
+int adamw_leaves(hipStream_t s, const olmax_leaf* leaves, int begin, int end, float* master, float* mom, float* var,
+                 bf16* shadow, const bf16* G, const float* grad_f32, int64_t step, float lr, float b1, float b2,
+                 float eps, float wd, int decay_embedding, const float* dscale) {
+  int i = begin;
+  while (i < end) {
+    const olmax_leaf& lf = leaves[i];
+    const float lwd = (lf.kind == OLMAX_LEAF_EMBEDDING && !decay_embedding) ? 0.f : wd;
+    if (lf.grad_f32) {
+      RC(olmax_adamw_dscale(s, master + lf.offset, grad_f32 + lf.grad_f32_offset, mom + lf.offset, var + lf.offset,
+                            shadow + lf.offset, lf.numel, 0, lr, b1, b2, eps, lwd, step, 1.f, dscale));
+      i++;
+    } else {
+      int64_t n = lf.numel;
+      int j = i + 1;
+      while (j < end && !leaves[j].grad_f32 && leaves[j].offset == lf.offset + n) {
+        n += leaves[j].numel;
+        j++;
+      }
+      RC(olmax_adamw_dscale(s, master + lf.offset, G + lf.offset, mom + lf.offset, var + lf.offset, shadow + lf.offset, n,
+                            1, lr, b1, b2, eps, lwd, step, 1.f, dscale));
+      i = j;
+    }
+  }
+  return OLMAX_OK;
+}
+
+// state of one overlapped train step: AdamW of a leaf group is launched on `opt` as soon as
+// the main stream has produced its gradients
+struct OverlapCtx {
+  hipStream_t main, opt;
+  hipEvent_t ev;
+  const olmax_leaf* leaves;
+  int nleaf;
+  float *master, *mom, *var;
+  bf16* shadow;
+  const bf16* G;
+  const float* grad_f32;
+  int64_t step;
+  float lr, b1, b2, eps, wd;
+  int decay_embedding;
+};
+int overlap_ready(void* vctx, int layer) {
+  OverlapCtx* x = (OverlapCtx*)vctx;
+  int begin = -1, end = -1;
+  for (int i = 0; i < x->nleaf; i++) {
+    const olmax_leaf& lf = x->leaves[i];
+    const bool in = layer >= 0 ? lf.layer == layer
+                   : layer == -1 ? (lf.kind == OLMAX_LEAF_FINAL_NORM || lf.kind == OLMAX_LEAF_LM_HEAD)
+                                 : lf.kind == OLMAX_LEAF_EMBEDDING;
+    if (in) {
+      if (begin < 0) begin = i;
+      end = i + 1;
+    }
+  }
+  if (begin < 0) return OLMAX_OK;
+  if (hipEventRecord(x->ev, x->main) != hipSuccess || hipStreamWaitEvent(x->opt, x->ev, 0) != hipSuccess)
+    return olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_model_train_step: event record/wait failed");
+  return adamw_leaves(x->opt, x->leaves, begin, end, x->master, x->mom, x->var, x->shadow, x->G, x->grad_f32, x->step, x->lr,
+                      x->b1, x->b2, x->eps, x->wd, x->decay_embedding, nullptr);
 }
 
 __global__ void clip_scale_kernel(const float* sumsq, float max_norm, float* out) {
@@ -591,27 +666,54 @@ extern "C" int32_t olmax_model_adamw(hipStream_t s, const olmax_model_config* c,
       dscale = norm_scratch;
     }
   }
-  // merge runs of adjacent bf16-gradient leaves (same decay) into single launches
-  int i = 0;
-  while (i < nleaf && !rc) {
-    const olmax_leaf& lf = leaves[i];
-    const float lwd = (lf.kind == OLMAX_LEAF_EMBEDDING && !decay_embedding) ? 0.f : wd;
-    if (lf.grad_f32) {
-      rc = olmax_adamw_dscale(s, master + lf.offset, grad_f32 + lf.grad_f32_offset, mom + lf.offset, var + lf.offset,
-                              shadow + lf.offset, lf.numel, 0, lr, b1, b2, eps, lwd, step, 1.f, dscale);
-      i++;
-    } else {
-      int64_t n = lf.numel;
-      int j = i + 1;
-      while (j < nleaf && !leaves[j].grad_f32 && leaves[j].offset == lf.offset + n) {
-        n += leaves[j].numel;
-        j++;
-      }
-      rc = olmax_adamw_dscale(s, master + lf.offset, G + lf.offset, mom + lf.offset, var + lf.offset, shadow + lf.offset,
-                              n, 1, lr, b1, b2, eps, lwd, step, 1.f, dscale);
-      i = j;
-    }
+  if (!rc) rc = adamw_leaves(s, leaves, 0, nleaf, master, mom, var, shadow, G, grad_f32, step, lr, b1, b2, eps, wd, decay_embedding, dscale);
+  delete[] leaves;
+  return rc;
+}
+
+// One micro-batch of training: loss + gradients, then AdamW.  With a second stream and no
+// gradient clipping the optimizer update of each layer (HBM-bound) runs on `opt_stream`
+// concurrently with the backward pass of the layers below it (MFMA-bound); `stream` waits for
+// the optimizer stream before returning control to later work.  Both streams must have the
+// default priority.  opt_stream == NULL (or clipping on) gives the plain sequence.
+extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_stream, const olmax_model_config* c,
+                                          const int32_t* windows, const float* const* cos_tables,
+                                          const float* const* sin_tables, float* master, float* mom, float* var,
+                                          void* params_bf16, const int32_t* ids, const int32_t* labels, float* loss,
+                                          void* grad_bf16, float* grad_f32, void* workspace, int64_t workspace_bytes,
+                                          int64_t step, float lr, float b1, float b2, float eps, float wd,
+                                          int32_t decay_embedding, float max_grad_norm, float* norm_scratch) {
+  RC(check_cfg(c));
+  OLMAX_CHECK(master && mom && var && params_bf16 && grad_bf16 && grad_f32, OLMAX_ERR_ARG, "olmax_model_train_step: null pointer");
+  OLMAX_CHECK(step >= 1, OLMAX_ERR_ARG, "olmax_model_train_step: step is 1-based");
+  if (!opt_stream || opt_stream == stream || max_grad_norm > 0.f) {
+    RC(model_run(stream, c, windows, cos_tables, sin_tables, params_bf16, ids, labels, loss, grad_bf16, grad_f32, workspace,
+                 workspace_bytes, true));
+    return olmax_model_adamw(stream, c, master, mom, var, params_bf16, grad_bf16, grad_f32, step, lr, b1, b2, eps, wd,
+                             decay_embedding, max_grad_norm, norm_scratch);
   }
+  // one event per thread, created on first use and kept for the life of the process
+  static thread_local hipEvent_t ev = nullptr;
+  if (!ev && hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess)
+    return olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_model_train_step: cannot create an event");
+  const int nleaf = olmax_model_layout(c, nullptr, 0);
+  olmax_leaf* leaves = new olmax_leaf[nleaf];
+  olmax_model_layout(c, leaves, nleaf);
+  OverlapCtx x{stream, opt_stream, ev, leaves, nleaf, master, mom, var, (bf16*)params_bf16, (const bf16*)grad_bf16, grad_f32,
+               step, lr, b1, b2, eps, wd, decay_embedding};
+  // the optimizer stream must not run ahead of work already queued on the main stream
+  int rc = OLMAX_OK;
+  if (hipEventRecord(ev, stream) != hipSuccess || hipStreamWaitEvent(opt_stream, ev, 0) != hipSuccess)
+    rc = olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_model_train_step: event record/wait failed");
+  GradReady ready;
+  ready.fn = overlap_ready;
+  ready.ctx = &x;
+  if (!rc)
+    rc = model_run(stream, c, windows, cos_tables, sin_tables, params_bf16, ids, labels, loss, grad_bf16, grad_f32, workspace,
+                   workspace_bytes, true, ready);
+  // join: later work on `stream` (the next step) sees every updated parameter
+  if (hipEventRecord(ev, opt_stream) != hipSuccess || hipStreamWaitEvent(stream, ev, 0) != hipSuccess)
+    rc = rc ? rc : olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_model_train_step: join failed");
   delete[] leaves;
   return rc;
 }

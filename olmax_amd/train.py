@@ -12,20 +12,20 @@ from .transformer import Transformer
 class Trainer:
     """Minimal step driver: loss + grads, then the fused AdamW update, once per micro-batch."""
 
-    def __init__(self, model: Transformer, optim: AdamWConfig):
+    def __init__(self, model: Transformer, optim: AdamWConfig, overlap_optimizer: bool = True):
         self.model, self.optim = model, optim
+        self.overlap_optimizer = overlap_optimizer
         self.count = 0  # optimizer steps taken
         self._decay_embedding = optim.decay_embedding()
         model.init_optimizer_state()
 
     def process_microbatch(self, input_ids: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
         lr = self.optim.lr_at(self.count)
-        loss = self.model.loss_and_grads(input_ids, labels)
         self.count += 1
-        self.model.adamw_step(step=self.count, lr=lr, b1=self.optim.b1, b2=self.optim.b2, eps=self.optim.eps,
-                              weight_decay=self.optim.weight_decay, decay_embedding=self._decay_embedding,
-                              max_grad_norm=self.optim.max_grad_norm)
-        return loss
+        return self.model.train_step(input_ids, labels, step=self.count, lr=lr, b1=self.optim.b1, b2=self.optim.b2,
+                                     eps=self.optim.eps, weight_decay=self.optim.weight_decay,
+                                     decay_embedding=self._decay_embedding, max_grad_norm=self.optim.max_grad_norm,
+                                     overlap_optimizer=self.overlap_optimizer)
 
     @property
     def grad_norm(self) -> Optional[float]:

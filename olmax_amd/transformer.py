@@ -210,6 +210,7 @@ class Transformer:
         self.loss = torch.zeros((), device=dev, dtype=torch.float32)
         self.norm_scratch = torch.zeros(2, device=dev, dtype=torch.float32)
         self._workspace: Optional[torch.Tensor] = None
+        self._opt_stream = None
 
         # per-layer windows and RoPE tables (get_buffer_cache, model.py:138-144)
         self._windows = (ctypes.c_int32 * max(1, config.num_layers))(*config.windows())
@@ -297,6 +298,28 @@ class Transformer:
         check(self._L.olmax_model_loss(
             stream_ptr(), ctypes.byref(self.c), self._windows, self._cos, self._sin, ptr(self.params_bf16),
             ptr(ids), ptr(labels), ptr(self.loss), ptr(ws), i64(ws.numel())))
+        return self.loss
+
+    def train_step(self, ids: torch.Tensor, labels: torch.Tensor, *, step: int, lr: float, b1: float = 0.9,
+                   b2: float = 0.999, eps: float = 1e-8, weight_decay: float = 1e-4, decay_embedding: bool = True,
+                   max_grad_norm: Optional[float] = None, overlap_optimizer: bool = True) -> torch.Tensor:
+        """loss + gradients + AdamW in one library call (process_microbatch).  With
+        ``overlap_optimizer`` each layer's AdamW runs on a second (default-priority) stream while
+        the backward pass continues."""
+        self._check_batch(ids, labels)
+        if self.m is None:
+            self.init_optimizer_state()
+        ws = self.workspace()
+        opt = None
+        if overlap_optimizer and not max_grad_norm:
+            if self._opt_stream is None:
+                self._opt_stream = torch.cuda.Stream(device=self.device)
+            opt = ctypes.c_void_p(self._opt_stream.cuda_stream)
+        check(self._L.olmax_model_train_step(
+            stream_ptr(), opt, ctypes.byref(self.c), self._windows, self._cos, self._sin, ptr(self.master), ptr(self.m),
+            ptr(self.v), ptr(self.params_bf16), ptr(ids), ptr(labels), ptr(self.loss), ptr(self.grad_bf16),
+            ptr(self.grad_f32), ptr(ws), i64(ws.numel()), i64(step), f32(lr), f32(b1), f32(b2), f32(eps),
+            f32(weight_decay), i32(int(decay_embedding)), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
         return self.loss
 
     def init_optimizer_state(self) -> None:

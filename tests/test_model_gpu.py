@@ -184,3 +184,29 @@ def test_single_block_fwd_bwd(kind):
     assert cosine(dx, wdx) >= 0.999
     for n, g in blk.grads.items():
         assert cosine(g, G["layers.0." + n]) >= 0.999, n
+
+
+def test_overlapped_optimizer_equals_sequential():
+    """AdamW launched per layer on a second stream during the backward pass gives the same
+    parameters as loss_and_grads followed by the whole-model AdamW."""
+    say("overlapped optimizer == sequential")
+    from olmax_amd import AdamWConfig, ConstantSchedule, Trainer
+    ocfg, hcfg = _cfgs("gemma")
+    B, S = 2, 128
+    P = _params(ocfg)
+    outs = []
+    for overlap in (False, True):
+        model = hcfg.build(batch_size=B, sequence_length=S)
+        model.load_state_dict(P)
+        tr = Trainer(model, AdamWConfig(lr=ConstantSchedule(1e-3), weight_decay=0.1), overlap_optimizer=overlap)
+        losses = []
+        for step in range(3):
+            gen = torch.Generator().manual_seed(step)
+            ids = torch.randint(0, 512, (B * S,), generator=gen, dtype=torch.int32).cuda()
+            labels = torch.randint(0, 512, (B * S,), generator=gen, dtype=torch.int32).cuda()
+            losses.append(tr.process_microbatch(ids, labels).item())
+        torch.cuda.synchronize()
+        outs.append((losses, model.master.clone(), model.params_bf16.clone()))
+    assert outs[0][0] == pytest.approx(outs[1][0], rel=1e-5)
+    assert relerr(outs[1][1], outs[0][1]) < 1e-5
+    assert (outs[0][2].float() - outs[1][2].float()).abs().max() <= 1e-2 * outs[0][2].float().abs().max()
