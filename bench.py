@@ -19,6 +19,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16 = 2.5e15  # dense MFMA bf16 FLOP/s of one MI355X
+# HBM-side bytes per launch of the dominant kernel (fetch + write, averaged over its 129 launches
+# per step), from the two rocprofv3 --pmc runs summarised in
+# profiles/gemm_traffic_pmc_llama7b_shapes.txt (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after
+# calibration against kernels of known size).
+GEMM_NT_TRAFFIC_BYTES = 2.06e9
+GEMM_NT_ALGORITHMIC_BYTES = 481 * 2 ** 20
 
 
 def cpu_baseline(sample_tokens: int = 512):
@@ -63,6 +69,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-checkpoint", action="store_true", help="keep activations instead of full-block recompute")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-keep-activations-leg", action="store_true", help="skip the extra measurement without recompute")
     ap.add_argument("--no-overlap", action="store_true", help="run AdamW after the backward pass instead of overlapping it on a second stream")
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline metric)")
     args = ap.parse_args()
@@ -133,7 +140,9 @@ def main():
     roofline = None
     if dom:
         roofline = {"bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s",
-                    "frac": dom["tflops"] / (PEAK_BF16 / 1e12), "traffic": None, "kernel": dom["kernel"],
+                    "frac": dom["tflops"] / (PEAK_BF16 / 1e12),
+                    "traffic": GEMM_NT_TRAFFIC_BYTES if dom["kernel"].endswith("A_KC,B_KC>") and cfg.num_layers == 32 else None,
+                    "algorithmic_bytes": GEMM_NT_ALGORITHMIC_BYTES, "kernel": dom["kernel"],
                     "avg_launch_ms": dom["avg_ms"], "launches_per_step": dom["launches"],
                     "all_gemm": {"ms_per_step": gemm_ms, "tflops": gemm_fl / gemm_ms if gemm_ms else None,
                                  "share_of_step": gemm_ms / ms_per_step}}
@@ -152,6 +161,24 @@ def main():
         "roofline": roofline,
         "gemm_kernels": per[:6],
     }
+    if not args.no_checkpoint and not args.no_keep_activations_leg:
+        # Same model, same step, but every block keeps its activations (34.8 GB of the 288 GB)
+        # instead of recomputing them: reported beside the headline value, never as it.
+        model.c.checkpoint = 0
+        model._workspace = None
+        torch.cuda.empty_cache()
+        for i in range(max(1, args.warmup)):
+            trainer.process_microbatch(*batches[i % nb])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            trainer.process_microbatch(*batches[i % nb])
+        torch.cuda.synchronize()
+        dt2 = time.perf_counter() - t0
+        tps2 = T * args.steps / dt2
+        out["keep_activations"] = {"value": tps2, "unit": "tokens/s", "ms_per_step": dt2 / args.steps * 1e3,
+                                   "mfu_bf16": tps2 * flops_tok / PEAK_BF16,
+                                   "note": "activation_checkpointing off (reference recipe default); not the headline config"}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
