@@ -156,76 +156,127 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
   // board's power limit (less accumulator traffic per FLOP).
   const int l16 = lane & 15, g16 = lane >> 4;
 
-  auto step = [&](const unsigned char* sa, const unsigned char* sb, int kk) {  // kk: 32-wide k-step
-    bf16x8 af[TM], bfr[TN];
+  // one operand fragment (16 rows x 32 k) of k-step kk (0 or 1) of a stage
+  auto load_a1 = [&](const unsigned char* sa, int kk, int i) -> bf16x8 {
+    if (A_KC) {
+      const int row = wm * WM + i * 16 + l16;
+      const int ch = kk * 4 + g16;
+      return *reinterpret_cast<const bf16x8*>(sa + row * 128 + ((ch ^ kswz(row)) << 4));
+    } else {
+      // transposing read: the 16-lane group g16 fetches k-rows kk*32 + 8*g16 + {0..3, 4..7}
+      const int col = wm * WM + i * 16 + ((l16 & 3) << 2);
+      Pack8 p;
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-      if (A_KC) {
-        const int row = wm * WM + i * 16 + l16;
-        const int ch = kk * 4 + g16;
-        af[i] = *reinterpret_cast<const bf16x8*>(sa + row * 128 + ((ch ^ kswz(row)) << 4));
-      } else {
-        // transposing read: the 16-lane group g16 fetches k-rows kk*32 + 8*g16 + {0..3, 4..7}
-        const int col = wm * WM + i * 16 + ((l16 & 3) << 2);
-        Pack8 p;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          const int kr = kk * 32 + g16 * 8 + h * 4 + (l16 >> 2);
-          const int off = kr * (BM * 2) + (((col >> 3) ^ tswz(kr)) << 4) + ((col & 7) << 1);
-          s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (s16x4 __attribute__((address_space(3)))*)(sa + off));
-          p.u[h * 2 + 0] = ((u32x2&)t)[0];
-          p.u[h * 2 + 1] = ((u32x2&)t)[1];
-        }
-        af[i] = p.v;
+      for (int h = 0; h < 2; h++) {
+        const int kr = kk * 32 + g16 * 8 + h * 4 + (l16 >> 2);
+        const int off = kr * (BM * 2) + (((col >> 3) ^ tswz(kr)) << 4) + ((col & 7) << 1);
+        s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4 __attribute__((address_space(3)))*)(sa + off));
+        p.u[h * 2 + 0] = ((u32x2&)t)[0];
+        p.u[h * 2 + 1] = ((u32x2&)t)[1];
       }
+      return p.v;
     }
+  };
+  auto load_b1 = [&](const unsigned char* sb, int kk, int j) -> bf16x8 {
+    if (B_KC) {
+      const int row = wn * WN + j * 16 + l16;
+      const int ch = kk * 4 + g16;
+      return *reinterpret_cast<const bf16x8*>(sb + row * 128 + ((ch ^ kswz(row)) << 4));
+    } else {
+      const int col = wn * WN + j * 16 + ((l16 & 3) << 2);
+      Pack8 p;
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-      if (B_KC) {
-        const int row = wn * WN + j * 16 + l16;
-        const int ch = kk * 4 + g16;
-        bfr[j] = *reinterpret_cast<const bf16x8*>(sb + row * 128 + ((ch ^ kswz(row)) << 4));
-      } else {
-        const int col = wn * WN + j * 16 + ((l16 & 3) << 2);
-        Pack8 p;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          const int kr = kk * 32 + g16 * 8 + h * 4 + (l16 >> 2);
-          const int off = kr * (BN * 2) + (((col >> 3) ^ tswz(kr)) << 4) + ((col & 7) << 1);
-          s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (s16x4 __attribute__((address_space(3)))*)(sb + off));
-          p.u[h * 2 + 0] = ((u32x2&)t)[0];
-          p.u[h * 2 + 1] = ((u32x2&)t)[1];
-        }
-        bfr[j] = p.v;
+      for (int h = 0; h < 2; h++) {
+        const int kr = kk * 32 + g16 * 8 + h * 4 + (l16 >> 2);
+        const int off = kr * (BN * 2) + (((col >> 3) ^ tswz(kr)) << 4) + ((col & 7) << 1);
+        s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4 __attribute__((address_space(3)))*)(sb + off));
+        p.u[h * 2 + 0] = ((u32x2&)t)[0];
+        p.u[h * 2 + 1] = ((u32x2&)t)[1];
       }
+      return p.v;
     }
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-      for (int j = 0; j < TN; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
   };
 
+  // ---- main loop.  Software pipeline, all of it in registers and the two LDS stages:
+  //   * fragments are double-buffered (fa/fb[0] = k-step 0, [1] = k-step 1 of a k-tile), and
+  //     every LDS read is issued half a k-tile before the MFMAs that consume it;
+  //   * the DMA of k-tile kt+2 goes into the stage k-tile kt occupied, right after the barrier
+  //     that retires it, so it has a whole k-tile of MFMAs to land;
+  //   * reads and DMA issues are slotted one per MFMA (pinned with sched_barrier), so that a
+  //     wave never leaves the matrix pipe without work for longer than one MFMA;
+  //   * the steady state has no branches: past the end the DMA re-fetches the last k-tile and
+  //     the reads fetch a stage nobody uses any more.
+  constexpr int NM = TM * TN, NF = TM + TN;
+  static_assert(2 * NINS <= NM && 2 * NF <= NM, "not enough MFMA slots for the loads");
+  bf16x8 fa[2][TM], fb[2][TN];
   dma(0, 0, 0, NINS);
-  dma_wait_all();
+  if (KT > 1) {
+    dma(1, 1, 0, NINS);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NINS) : "memory");  // k-tile 0 has landed
+  } else {
+    dma_wait_all();
+  }
   __syncthreads();
+#pragma unroll
+  for (int i = 0; i < TM; i++) fa[0][i] = load_a1(smem, 0, i);
+#pragma unroll
+  for (int j = 0; j < TN; j++) fb[0][j] = load_b1(smem + A_BYTES, 0, j);
+  // running DMA sources: k-tile kt+2 while it exists, then they stop advancing
+  const bf16* ap[A_INS];
+  const bf16* bp[B_INS];
+  {
+    const int k2 = min(2, KT - 1);
+#pragma unroll
+    for (int i = 0; i < A_INS; i++) ap[i] = a_src[i] + (int64_t)k2 * a_step;
+#pragma unroll
+    for (int i = 0; i < B_INS; i++) bp[i] = b_src[i] + (int64_t)k2 * b_step;
+  }
   for (int kt = 0; kt < KT; kt++) {
     const int cur = kt & 1;
     const unsigned char* sa = smem + cur * STAGE;
     const unsigned char* sb = sa + A_BYTES;
-    const bool more = kt + 1 < KT;
+    const unsigned char* na = smem + (cur ^ 1) * STAGE;
+    const unsigned char* nb = na + A_BYTES;
+    const unsigned da = lds_base + cur * STAGE, db = da + A_BYTES;
+    const int64_t adv_a = (kt + 3 < KT) ? a_step : 0, adv_b = (kt + 3 < KT) ? b_step : 0;
+    // k-step 0 from registers; the fragments of k-step 1 are fetched meanwhile
 #pragma unroll
-    for (int kk = 0; kk < BK / 32; kk++) {
-      // the next k-tile streams into the other stage while this one is consumed; its DMA
-      // instructions are spread over the k-steps so that no wave stalls on a full queue
-      if (more) dma(kt + 1, cur ^ 1, kk * NINS / 2, (kk + 1) * NINS / 2);
-      step(sa, sb, kk);
+    for (int m = 0; m < NM; m++) {
+      const int i = m / TN, j = m % TN;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
+      if (m < TN) fb[1][m] = load_b1(sb, 1, m);
+      else if (m < NF) fa[1][m - TN] = load_a1(sa, 1, m - TN);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    dma_wait_all();
+    // k-tile kt+1 has landed (issued one k-tile ago); every wave is done reading k-tile kt
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
+    // k-step 1 from registers; even slots issue the DMA of k-tile kt+2 into the retired stage,
+    // odd slots fetch k-step 0 of k-tile kt+1
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+      const int i = m / TN, j = m % TN;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
+      if ((m & 1) == 0 && (m >> 1) < NINS) {
+        const int q = m >> 1;
+        if (q < A_INS) {
+          dma16(ap[q], da + (q * NW + wave) * 1024);
+          ap[q] += adv_a;
+        } else {
+          dma16(bp[q - A_INS], db + ((q - A_INS) * NW + wave) * 1024);
+          bp[q - A_INS] += adv_b;
+        }
+      } else if ((m & 1) == 1 && (m >> 1) < NF) {
+        const int f = m >> 1;
+        if (f < TN) fb[0][f] = load_b1(nb, 0, f);
+        else fa[0][f - TN] = load_a1(na, 0, f - TN);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
+  dma_wait_all();  // the redundant tail DMAs must not outlive the workgroup's LDS allocation
 
   // ---- epilogue: accumulator lane -> column l16, rows 4*g16 + r of each 16x16 tile
 #pragma unroll
