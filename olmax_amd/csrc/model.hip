@@ -733,7 +733,7 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
   olmax_leaf* leaves = new olmax_leaf[nleaf];
   olmax_model_layout(c, leaves, nleaf);
   OverlapCtx x{stream, opt_stream, ev, leaves, nleaf, master, mom, var, (bf16*)params_bf16, (const bf16*)grad_bf16, grad_f32,
-               step, lr, b1, b2, eps, wd, decay_embedding, POINT_RECOMPUTE_ATTN, {0, 0, 0, 0}, 0};
+               step, lr, b1, b2, eps, wd, decay_embedding, c->checkpoint ? POINT_RECOMPUTE_ATTN : POINT_ATTN_BWD, {0, 0, 0, 0}, 0};
   // the optimizer stream must not run ahead of work already queued on the main stream
   int rc = OLMAX_OK;
   if (hipEventRecord(ev, stream) != hipSuccess || hipStreamWaitEvent(opt_stream, ev, 0) != hipSuccess)
