@@ -110,6 +110,50 @@ __device__ __forceinline__ void dma_tile(const bf16* base, int64_t ld, int r0, i
   }
 }
 
+// Workgroup id -> (tile rank, K/V group, head inside the group).  Hardware deals consecutive
+// ids round-robin to the 8 XCDs and every XCD starts its ids in order, so the tile rank (the
+// amount of causal work) is the SLOWEST index: each XCD gets the same mix of long and short
+// tiles and starts the longest first (with the rank fastest, one XCD got 54 % more work than
+// another and the CUs idled 39 % of the kernel).  When the group count divides by 8 the
+// heads sharing a K/V head also land on one XCD, i.e. one L2.
+struct WgCoord { int rank, group, r; };
+__device__ __forceinline__ WgCoord decode_wg(int id, int ngroups, int rep) {
+  const int level = ngroups * rep;
+  WgCoord c;
+  c.rank = id / level;
+  const int u = id % level;
+  if ((ngroups & 7) == 0) {
+    const int blk = u / (8 * rep), rem = u % (8 * rep);
+    c.r = rem >> 3;
+    c.group = blk * 8 + (rem & 7);
+  } else {
+    c.group = u / rep;
+    c.r = u % rep;
+  }
+  return c;
+}
+
+// The same tile transfer with everything lane-dependent hoisted out of the loop: per-lane
+// byte offsets (row * ld + swizzled chunk) are computed once, a transfer is ROWS/16 DMA
+// instructions off a wave-uniform row pointer.  Only for tiles that lie entirely inside the
+// sequence (no row clamping).
+template <int ROWS>
+struct TileDma {
+  unsigned off[ROWS / 16];
+  __device__ __forceinline__ void init(int64_t ld, int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < ROWS / 16; i++) {
+      const int p = (i * 4 + wave) * 64 + lane;
+      const int row = p >> 4, ph = p & 15;
+      off[i] = (unsigned)((row * ld + ((ph ^ swz(row)) << 3)) * 2);
+    }
+  }
+  __device__ __forceinline__ void issue(const bf16* row0, unsigned lds_addr, int wave) const {
+#pragma unroll
+    for (int i = 0; i < ROWS / 16; i++) dma16_s(row0, off[i], lds_addr + (i * 4 + wave) * 1024);
+  }
+};
+
 __device__ __forceinline__ bf16x8 pack_bf16x8(const f32x16& a, int base) {
   bf16x8 r;
 #pragma unroll
@@ -124,7 +168,7 @@ __device__ __forceinline__ float fast_tanh(float x) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Forward.  grid = (ceil(S/128), H, B); 256 threads; wave w owns queries i0+32w .. +31.
+// Forward.  grid = ceil(S/128)*H*B workgroups (see decode_wg); 256 threads; wave w owns queries i0+32w .. +31.
 // ---------------------------------------------------------------------------------------
 template <bool CAP>
 __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
@@ -134,9 +178,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [2][K 16K | V 16K]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
-  const int qt = gridDim.x - 1 - blockIdx.x;  // longest rows first
-  const int h = blockIdx.y, b = blockIdx.z;
-  const int kh = h / (H / KH);
+  const int nqt = (S + 127) >> 7;
+  const WgCoord wg = decode_wg(blockIdx.x, (int)(gridDim.x / (nqt * (H / KH))), H / KH);
+  const int qt = nqt - 1 - wg.rank;  // longest rows first
+  const int b = wg.group / KH, kh = wg.group % KH;
+  const int h = kh * (H / KH) + wg.r;
   const int i0 = qt * 128;
   const int iw0 = i0 + wave * 32;  // first query of this wave
   const int qi = iw0 + l32;        // this lane's query
@@ -163,9 +209,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
   const bf16* vbase = V + (int64_t)b * S * ldv + kh * 128;
   const unsigned lds0 = lds_addr_of(smem);
   const int wv = __builtin_amdgcn_readfirstlane(wave);
+  TileDma<64> dk, dv;
+  dk.init(ldk, wv, lane);
+  dv.init(ldv, wv, lane);
   auto load_kv = [&](int t, int stage) {
-    dma_tile<64>(kbase, ldk, t * 64, S, lds0 + stage * 32768, wv, lane);
-    dma_tile<64>(vbase, ldv, t * 64, S, lds0 + stage * 32768 + 16384, wv, lane);
+    if (t * 64 + 64 <= S) {
+      dk.issue(kbase + (int64_t)t * 64 * ldk, lds0 + stage * 32768, wv);
+      dv.issue(vbase + (int64_t)t * 64 * ldv, lds0 + stage * 32768 + 16384, wv);
+    } else {
+      dma_tile<64>(kbase, ldk, t * 64, S, lds0 + stage * 32768, wv, lane);
+      dma_tile<64>(vbase, ldv, t * 64, S, lds0 + stage * 32768 + 16384, wv, lane);
+    }
   };
   const float sc2 = scale * LOG2E;
   FragAddr fa;
@@ -298,7 +352,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------
-// dQ.  Same tiling as the forward: grid = (ceil(S/128), H, B); K/V tiles stream through LDS.
+// dQ.  Same tiling and grid as the forward; K/V tiles stream through LDS.
 // ---------------------------------------------------------------------------------------
 template <bool CAP>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
@@ -309,9 +363,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
-  const int qt = gridDim.x - 1 - blockIdx.x;
-  const int h = blockIdx.y, b = blockIdx.z;
-  const int kh = h / (H / KH);
+  const int nqt = (S + 127) >> 7;
+  const WgCoord wg = decode_wg(blockIdx.x, (int)(gridDim.x / (nqt * (H / KH))), H / KH);
+  const int qt = nqt - 1 - wg.rank;  // longest rows first
+  const int b = wg.group / KH, kh = wg.group % KH;
+  const int h = kh * (H / KH) + wg.r;
   const int i0 = qt * 128;
   const int iw0 = i0 + wave * 32;
   const int qi = iw0 + l32;
@@ -343,9 +399,17 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
   const bf16* vbase = V + (int64_t)b * S * ldv + kh * 128;
   const unsigned lds0 = lds_addr_of(smem);
   const int wv = __builtin_amdgcn_readfirstlane(wave);
+  TileDma<64> dk, dv;
+  dk.init(ldk, wv, lane);
+  dv.init(ldv, wv, lane);
   auto load_kv = [&](int t, int stage) {
-    dma_tile<64>(kbase, ldk, t * 64, S, lds0 + stage * 32768, wv, lane);
-    dma_tile<64>(vbase, ldv, t * 64, S, lds0 + stage * 32768 + 16384, wv, lane);
+    if (t * 64 + 64 <= S) {
+      dk.issue(kbase + (int64_t)t * 64 * ldk, lds0 + stage * 32768, wv);
+      dv.issue(vbase + (int64_t)t * 64 * ldv, lds0 + stage * 32768 + 16384, wv);
+    } else {
+      dma_tile<64>(kbase, ldk, t * 64, S, lds0 + stage * 32768, wv, lane);
+      dma_tile<64>(vbase, ldv, t * 64, S, lds0 + stage * 32768 + 16384, wv, lane);
+    }
   };
   const float sc2 = scale * LOG2E;
 
@@ -421,7 +485,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// dK/dV.  grid = (ceil(S/128), KH, B); wave w owns keys j0+32w..+31 (K and V fragments stay in
+// dK/dV.  grid = ceil(S/128)*KH*B workgroups; wave w owns keys j0+32w..+31 (K and V fragments stay in
 // registers); loops over the query heads of its group and over 32-row Q/dO tiles from the
 // diagonal downwards.  LDS: 2 stages of (Q 8K | dO 8K | lse 128 B | delta 128 B) + V tile 32K.
 // ---------------------------------------------------------------------------------------
@@ -436,8 +500,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
   constexpr int STAGE = 2 * QT * 256 + 256;  // Q | dO | lse, delta
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
-  const int kt = blockIdx.x;
-  const int kh = blockIdx.y, b = blockIdx.z;
+  // key tile 0 is seen by every query: rank order is already longest first
+  const WgCoord wg = decode_wg(blockIdx.x, (int)(gridDim.x / ((S + 127) >> 7)), 1);
+  const int kt = wg.rank;
+  const int b = wg.group / KH, kh = wg.group % KH;
   const int rep = H / KH;
   const int j0 = kt * 128;
   const int jw0 = j0 + wave * 32;
@@ -468,11 +534,19 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
   const int wv = __builtin_amdgcn_readfirstlane(wave);
 
   float sreg = 0.f;
+  TileDma<QT> tq, tdo;
+  tq.init(ldq, wv, lane);
+  tdo.init(lddo, wv, lane);
   auto load_tile = [&](int it, int stage) {
     const int hq = kh * rep + it / ntile;
     const int t = t_lo + it % ntile;
-    dma_tile<QT>(Q + (int64_t)b * S * ldq + hq * 128, ldq, t * QT, S, lds0 + stage * STAGE, wv, lane);
-    dma_tile<QT>(dO + (int64_t)b * S * lddo + hq * 128, lddo, t * QT, S, lds0 + stage * STAGE + QT * 256, wv, lane);
+    if (t * QT + QT <= S) {
+      tq.issue(Q + ((int64_t)b * S + t * QT) * ldq + hq * 128, lds0 + stage * STAGE, wv);
+      tdo.issue(dO + ((int64_t)b * S + t * QT) * lddo + hq * 128, lds0 + stage * STAGE + QT * 256, wv);
+    } else {
+      dma_tile<QT>(Q + (int64_t)b * S * ldq + hq * 128, ldq, t * QT, S, lds0 + stage * STAGE, wv, lane);
+      dma_tile<QT>(dO + (int64_t)b * S * lddo + hq * 128, lddo, t * QT, S, lds0 + stage * STAGE + QT * 256, wv, lane);
+    }
     if (tid < 2 * QT) {
       const int ii = min(t * QT + (tid & (QT - 1)), S - 1);
       const float* src = tid < QT ? LSE : DELTA;
@@ -700,7 +774,7 @@ extern "C" int32_t olmax_attn_fwd(hipStream_t stream, const void* q, const void*
   const float scale = 1.f / sqrtf((float)D);
   const bf16 *qp = (const bf16*)q, *kp = (const bf16*)k, *vp = (const bf16*)v;
   if (fast_ok(D, q, k, v, o, ldq, ldk, ldv, ldo)) {
-    dim3 grid((S + 127) / 128, H, B);
+    dim3 grid((unsigned)(((S + 127) / 128) * H * B));
     if (softcap > 0.f) {
       static bool set = false;
       if (!set) { (void)hipFuncSetAttribute((const void*)attn_fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536); set = true; }
@@ -744,7 +818,7 @@ extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void*
   if (fast) {
     const int64_t units = (int64_t)B * S * H;
     hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((units + 15) / 16)), dim3(256), 0, stream, op, gop, delta, B, S, H, ldo, lddo);
-    dim3 gkv((S + 127) / 128, KH, B), gq((S + 127) / 128, H, B);
+    dim3 gkv((unsigned)(((S + 127) / 128) * KH * B)), gq((unsigned)(((S + 127) / 128) * H * B));
     constexpr int SM_KV = 2 * (2 * 32 * 256 + 256) + 128 * 256;
     static bool set = false;
     if (!set) {

@@ -62,6 +62,11 @@ union Pack4 {
 __device__ __forceinline__ void dma16(const void* g, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(g) : "m0", "memory");
 }
+// Same, addressed as a wave-uniform 64-bit base (SGPR pair) plus a per-lane unsigned 32-bit
+// byte offset: a lane's offset inside a tile is loop invariant, only the base moves.
+__device__ __forceinline__ void dma16_s(const void* sbase, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "m0", "memory");
+}
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ unsigned lds_addr_of(const void* p) {
   return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)p;
