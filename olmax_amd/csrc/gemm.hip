@@ -410,6 +410,16 @@ extern "C" int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flo
   return n;
 }
 
+static int device_cu_count() {
+  static int n = 0;
+  if (!n) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n = v;
+    else n = 256;
+  }
+  return n;
+}
+
 extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void* B, void* C,
                                    const void* R, int32_t M, int32_t N, int32_t K, int64_t lda,
                                    int64_t ldb, int64_t ldc, int64_t ldr, int32_t a_layout,
@@ -433,6 +443,38 @@ extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void
   if (g_force_tile && tile) {
     if (g_force_tile == 256 && M % 256 == 0 && N % 256 == 0) tile = 256;
     if (g_force_tile == 128) tile = 128;
+  }
+  // Wave quantisation: with one 256x256 tile per CU per round, a last round that fills less
+  // than half of the CUs (e.g. 1376 tiles = 5.375 rounds on 256 CUs) costs a whole round.
+  // Such a problem is cut along M or N into a part whose tile count is a whole number of
+  // rounds and a remainder that goes through this function again (and gets smaller tiles).
+  if (tile == 256 && !g_force_tile) {
+    const int ncu = device_cu_count();
+    const int tm = M / 256, tn = N / 256;
+    const int64_t tiles = (int64_t)tm * tn;
+    const int rem = (int)(tiles % ncu);
+    if (tiles > ncu && rem > 0 && rem * 2 < ncu) {
+      int rm = 0, cn = 0;  // largest row-tile / column-tile counts giving whole rounds
+      for (int x = tm - 1; x > 0; x--) if (((int64_t)x * tn) % ncu == 0) { rm = x; break; }
+      for (int x = tn - 1; x > 0; x--) if (((int64_t)x * tm) % ncu == 0) { cn = x; break; }
+      const size_t esz = out_f32 ? 4 : 2;
+      if (rm > 0 && (int64_t)rm * tn >= (int64_t)cn * tm) {
+        const int m1 = rm * 256;
+        int rc = olmax_gemm_bf16(stream, A, B, C, R, m1, N, K, lda, ldb, ldc, ldr, a_layout, b_layout, out_f32);
+        if (rc) return rc;
+        const bf16* a2 = a_kc ? a + (int64_t)m1 * lda : a + m1;
+        return olmax_gemm_bf16(stream, a2, B, (char*)C + (int64_t)m1 * ldc * esz, r ? r + (int64_t)m1 * ldr : nullptr,
+                               M - m1, N, K, lda, ldb, ldc, ldr, a_layout, b_layout, out_f32);
+      }
+      if (cn > 0) {
+        const int n1 = cn * 256;
+        int rc = olmax_gemm_bf16(stream, A, B, C, R, M, n1, K, lda, ldb, ldc, ldr, a_layout, b_layout, out_f32);
+        if (rc) return rc;
+        const bf16* b2 = b_kc ? b + (int64_t)n1 * ldb : b + n1;
+        return olmax_gemm_bf16(stream, A, b2, (char*)C + (int64_t)n1 * esz, r ? r + n1 : nullptr, M, N - n1, K, lda,
+                               ldb, ldc, ldr, a_layout, b_layout, out_f32);
+      }
+    }
   }
   if (tile == 0) {
     dim3 grid((N + 15) / 16, (M + 15) / 16);
