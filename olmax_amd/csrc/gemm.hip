@@ -92,35 +92,37 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
   auto kswz = [](int row) { return (row >> 1) & 7; };                         // [rows][64] tiles
   auto tswz = [](int kr) { return ((kr & 3) << 2) | ((kr >> 2) & 2); };        // [64][rows] tiles
 
-  // ---- per-lane DMA sources: instruction i of this wave fills LDS block (i*NW + wave) of
-  // 1 KB, i.e. 16-byte chunks p = block*64 + lane of the tile; the lane fetches whichever
-  // global chunk the swizzle places there ----
-  const bf16* a_src[A_INS];
+  // ---- DMA sources: instruction i of this wave fills LDS block (i*NW + wave) of 1 KB, i.e.
+  // 16-byte chunks p = block*64 + lane of the tile; the lane fetches whichever global chunk the
+  // swizzle places there.  A lane's byte offset inside the operand panel never changes; the
+  // k-tile only moves the wave-uniform base (SGPRs), so the loop spends no VALU on addresses.
+  unsigned a_off[A_INS], b_off[B_INS];
 #pragma unroll
   for (int i = 0; i < A_INS; i++) {
     const int p = (i * NW + wave) * 64 + lane;
     if (A_KC) {
       const int row = p >> 3, ph = p & 7;
-      a_src[i] = A + (int64_t)(m0 + row) * lda + ((ph ^ kswz(row)) << 3);
+      a_off[i] = (unsigned)(((int64_t)row * lda + ((ph ^ kswz(row)) << 3)) * 2);
     } else {
       constexpr int CPR = BM / 8;  // chunks per k-row
       const int kr = p / CPR, ph = p % CPR;
-      a_src[i] = A + (int64_t)kr * lda + m0 + ((ph ^ tswz(kr)) << 3);
+      a_off[i] = (unsigned)(((int64_t)kr * lda + ((ph ^ tswz(kr)) << 3)) * 2);
     }
   }
-  const bf16* b_src[B_INS];
 #pragma unroll
   for (int i = 0; i < B_INS; i++) {
     const int p = (i * NW + wave) * 64 + lane;
     if (B_KC) {
       const int row = p >> 3, ph = p & 7;
-      b_src[i] = B + (int64_t)(n0 + row) * ldb + ((ph ^ kswz(row)) << 3);
+      b_off[i] = (unsigned)(((int64_t)row * ldb + ((ph ^ kswz(row)) << 3)) * 2);
     } else {
       constexpr int CPR = BN / 8;
       const int kr = p / CPR, ph = p % CPR;
-      b_src[i] = B + (int64_t)kr * ldb + n0 + ((ph ^ tswz(kr)) << 3);
+      b_off[i] = (unsigned)(((int64_t)kr * ldb + ((ph ^ tswz(kr)) << 3)) * 2);
     }
   }
+  const bf16* a_panel = A_KC ? A + (int64_t)m0 * lda : A + m0;  // k-tile 0 of this block's rows
+  const bf16* b_panel = B_KC ? B + (int64_t)n0 * ldb : B + n0;
   const int64_t a_step = A_KC ? (int64_t)BK : (int64_t)BK * lda;
   const int64_t b_step = B_KC ? (int64_t)BK : (int64_t)BK * ldb;
 
@@ -142,10 +144,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
     for (int i = 0; i < NINS; i++) {
       if (i < lo || i >= hi) continue;
       if (i < A_INS) {
-        dma16(a_src[i] + (int64_t)kt * a_step, sa + (i * NW + wave) * 1024);
+        dma16_s(a_panel + (int64_t)kt * a_step, a_off[i], sa + (i * NW + wave) * 1024);
       } else {
         const int j = i - A_INS;
-        dma16(b_src[j] + (int64_t)kt * b_step, sb + (j * NW + wave) * 1024);
+        dma16_s(b_panel + (int64_t)kt * b_step, b_off[j], sb + (j * NW + wave) * 1024);
       }
     }
   };
@@ -223,16 +225,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
   for (int i = 0; i < TM; i++) fa[0][i] = load_a1(smem, 0, i);
 #pragma unroll
   for (int j = 0; j < TN; j++) fb[0][j] = load_b1(smem + A_BYTES, 0, j);
-  // running DMA sources: k-tile kt+2 while it exists, then they stop advancing
-  const bf16* ap[A_INS];
-  const bf16* bp[B_INS];
-  {
-    const int k2 = min(2, KT - 1);
-#pragma unroll
-    for (int i = 0; i < A_INS; i++) ap[i] = a_src[i] + (int64_t)k2 * a_step;
-#pragma unroll
-    for (int i = 0; i < B_INS; i++) bp[i] = b_src[i] + (int64_t)k2 * b_step;
-  }
+  // running DMA bases: k-tile kt+2 while it exists, then they stop advancing
+  const bf16* ap = a_panel + (int64_t)min(2, KT - 1) * a_step;
+  const bf16* bp = b_panel + (int64_t)min(2, KT - 1) * b_step;
   for (int kt = 0; kt < KT; kt++) {
     const int cur = kt & 1;
     const unsigned char* sa = smem + cur * STAGE;
@@ -240,7 +235,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
     const unsigned char* na = smem + (cur ^ 1) * STAGE;
     const unsigned char* nb = na + A_BYTES;
     const unsigned da = lds_base + cur * STAGE, db = da + A_BYTES;
-    const int64_t adv_a = (kt + 3 < KT) ? a_step : 0, adv_b = (kt + 3 < KT) ? b_step : 0;
     // k-step 0 from registers; the fragments of k-step 1 are fetched meanwhile
 #pragma unroll
     for (int m = 0; m < NM; m++) {
@@ -261,19 +255,18 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
       acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
       if ((m & 1) == 0 && (m >> 1) < NINS) {
         const int q = m >> 1;
-        if (q < A_INS) {
-          dma16(ap[q], da + (q * NW + wave) * 1024);
-          ap[q] += adv_a;
-        } else {
-          dma16(bp[q - A_INS], db + ((q - A_INS) * NW + wave) * 1024);
-          bp[q - A_INS] += adv_b;
-        }
+        if (q < A_INS) dma16_s(ap, a_off[q], da + (q * NW + wave) * 1024);
+        else dma16_s(bp, b_off[q - A_INS], db + ((q - A_INS) * NW + wave) * 1024);
       } else if ((m & 1) == 1 && (m >> 1) < NF) {
         const int f = m >> 1;
         if (f < TN) fb[0][f] = load_b1(nb, 0, f);
         else fa[0][f - TN] = load_a1(na, 0, f - TN);
       }
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (kt + 3 < KT) {
+      ap += a_step;
+      bp += b_step;
     }
   }
   dma_wait_all();  // the redundant tail DMAs must not outlive the workgroup's LDS allocation
