@@ -230,9 +230,10 @@ int32_t olmax_model_adamw(olmax_stream_t stream, const olmax_model_config* cfg, 
                           float wd, int32_t decay_embedding, float max_grad_norm, float* norm_scratch);
 
 /* process_microbatch, src/olmax/train/trainer.py:759-777: loss + gradients + AdamW in one call.
- * opt_stream (optional, default priority, != stream): when given and clipping is off, each
- * layer's AdamW runs there concurrently with the backward pass of the layers below it, and
- * `stream` waits for it at the end.  Creates one HIP event per host thread on first use. */
+ * opt_stream (optional, default priority, != stream): when given, clipping is off and the config
+ * checkpoints its blocks, each layer's AdamW runs there concurrently with the recompute and
+ * backward of the layers below it, and `stream` waits for it at the end; otherwise AdamW follows
+ * the backward pass on `stream`.  Creates one HIP event per host thread on first use. */
 int32_t olmax_model_train_step(olmax_stream_t stream, olmax_stream_t opt_stream, const olmax_model_config* cfg,
                                const int32_t* windows, const float* const* cos_tables,
                                const float* const* sin_tables, float* master, float* m, float* v,

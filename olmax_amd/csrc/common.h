@@ -111,3 +111,8 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   for (int i = 1; i < NW; i++) t = fmaxf(t, red[i]);
   return t;
 }
+
+// elementwise.hip, library-internal: olmax_adamw_dscale with the grid size (workgroups) exposed.
+int olmax_adamw_grid(hipStream_t stream, float* p, const void* g, float* m, float* v, void* shadow_bf16, int64_t n,
+                     int32_t grad_is_bf16, float lr, float b1, float b2, float eps, float wd, int64_t step,
+                     float grad_scale, const float* grad_scale_dev, int grid_cap);

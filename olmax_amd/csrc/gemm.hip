@@ -39,6 +39,10 @@ namespace {
 
 constexpr int BK = 64;
 
+#ifndef GEMM_VGPR_CAP
+#define GEMM_VGPR_CAP
+#endif
+
 // Optional per-launch timing (HIP events recorded on the launch stream around every GEMM),
 // switched on by olmax_gemm_profile_begin(); used by the benchmark's roofline report.
 struct ProfRec {
@@ -51,7 +55,7 @@ std::vector<ProfRec> g_prof;
 std::mutex g_prof_mu;
 
 template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_bf16_kernel(
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm_bf16_kernel(
     const bf16* __restrict__ A, const bf16* __restrict__ B, void* __restrict__ Cv,
     const bf16* __restrict__ R, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
     int64_t ldr, int tiles_m, int tiles_n) {

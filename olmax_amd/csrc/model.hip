@@ -470,14 +470,14 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
 // the same decay become single launches.
 int adamw_leaves(hipStream_t s, const olmax_leaf* leaves, int begin, int end, float* master, float* mom, float* var,
                  bf16* shadow, const bf16* G, const float* grad_f32, int64_t step, float lr, float b1, float b2,
-                 float eps, float wd, int decay_embedding, const float* dscale) {
+                 float eps, float wd, int decay_embedding, const float* dscale, int grid_cap = 512) {
   int i = begin;
   while (i < end) {
     const olmax_leaf& lf = leaves[i];
     const float lwd = (lf.kind == OLMAX_LEAF_EMBEDDING && !decay_embedding) ? 0.f : wd;
     if (lf.grad_f32) {
-      RC(olmax_adamw_dscale(s, master + lf.offset, grad_f32 + lf.grad_f32_offset, mom + lf.offset, var + lf.offset,
-                            shadow + lf.offset, lf.numel, 0, lr, b1, b2, eps, lwd, step, 1.f, dscale));
+      RC(olmax_adamw_grid(s, master + lf.offset, grad_f32 + lf.grad_f32_offset, mom + lf.offset, var + lf.offset,
+                          shadow + lf.offset, lf.numel, 0, lr, b1, b2, eps, lwd, step, 1.f, dscale, grid_cap));
       i++;
     } else {
       int64_t n = lf.numel;
@@ -486,8 +486,8 @@ int adamw_leaves(hipStream_t s, const olmax_leaf* leaves, int begin, int end, fl
         n += leaves[j].numel;
         j++;
       }
-      RC(olmax_adamw_dscale(s, master + lf.offset, G + lf.offset, mom + lf.offset, var + lf.offset, shadow + lf.offset, n,
-                            1, lr, b1, b2, eps, lwd, step, 1.f, dscale));
+      RC(olmax_adamw_grid(s, master + lf.offset, G + lf.offset, mom + lf.offset, var + lf.offset, shadow + lf.offset, n, 1,
+                          lr, b1, b2, eps, lwd, step, 1.f, dscale, grid_cap));
       i = j;
     }
   }
@@ -508,10 +508,11 @@ struct OverlapCtx {
   int64_t step;
   float lr, b1, b2, eps, wd;
   int decay_embedding;
-  // 0: launch as soon as the gradients are final; else at that StepHook point.  The big
-  // kernels fill every CU's register file, so the optimizer never truly shares a CU with
-  // them; starting it next to the recomputed attention (the least matrix-bound stretch of a
-  // block) measured best (about 1 % of the 7B step over launching at once).
+  // 0: launch as soon as the gradients are final; else at that StepHook point.  Measured on
+  // the 7B step: AdamW as a one-workgroup-per-CU grid of 32-register waves launched at once
+  // (it then shares CUs with the next block's forward GEMMs, whose waves leave it 32 registers
+  // per lane) gains 1.3 % over the sequential step; deferring it to an attention kernel (whose
+  // waves fill the register file, so the two only time-slice) loses 5 %.
   int flush_point;
   int pending[4];      // leaf groups whose gradients are final but whose AdamW is not launched yet
   int npending;
@@ -547,7 +548,7 @@ int overlap_launch(OverlapCtx* x, int layer) {
   if (hipEventRecord(x->ev, x->main) != hipSuccess || hipStreamWaitEvent(x->opt, x->ev, 0) != hipSuccess)
     return olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_model_train_step: event record/wait failed");
   return adamw_leaves(x->opt, x->leaves, begin, end, x->master, x->mom, x->var, x->shadow, x->G, x->grad_f32, x->step, x->lr,
-                      x->b1, x->b2, x->eps, x->wd, x->decay_embedding, nullptr);
+                      x->b1, x->b2, x->eps, x->wd, x->decay_embedding, nullptr, 256);
 }
 
 __global__ void clip_scale_kernel(const float* sumsq, float max_norm, float* out) {
@@ -719,7 +720,9 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
   RC(check_cfg(c));
   OLMAX_CHECK(master && mom && var && params_bf16 && grad_bf16 && grad_f32, OLMAX_ERR_ARG, "olmax_model_train_step: null pointer");
   OLMAX_CHECK(step >= 1, OLMAX_ERR_ARG, "olmax_model_train_step: step is 1-based");
-  if (!opt_stream || opt_stream == stream || max_grad_norm > 0.f) {
+  // Without recompute the optimizer would share the GPU with the backward GEMMs only (no
+  // forward GEMMs in between), which measured 4 % slower than running it afterwards.
+  if (!opt_stream || opt_stream == stream || max_grad_norm > 0.f || !c->checkpoint) {
     RC(model_run(stream, c, windows, cos_tables, sin_tables, params_bf16, ids, labels, loss, grad_bf16, grad_f32, workspace,
                  workspace_bytes, true));
     return olmax_model_adamw(stream, c, master, mom, var, params_bf16, grad_bf16, grad_f32, step, lr, b1, b2, eps, wd,
@@ -733,7 +736,7 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
   olmax_leaf* leaves = new olmax_leaf[nleaf];
   olmax_model_layout(c, leaves, nleaf);
   OverlapCtx x{stream, opt_stream, ev, leaves, nleaf, master, mom, var, (bf16*)params_bf16, (const bf16*)grad_bf16, grad_f32,
-               step, lr, b1, b2, eps, wd, decay_embedding, c->checkpoint ? POINT_RECOMPUTE_ATTN : POINT_ATTN_BWD, {0, 0, 0, 0}, 0};
+               step, lr, b1, b2, eps, wd, decay_embedding, 0, {0, 0, 0, 0}, 0};
   // the optimizer stream must not run ahead of work already queued on the main stream
   int rc = OLMAX_OK;
   if (hipEventRecord(ev, stream) != hipSuccess || hipStreamWaitEvent(opt_stream, ev, 0) != hipSuccess)
