@@ -89,12 +89,12 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_generic(const bf16* __restric
 // ------------------------------------------------------------------ RMSNorm backward
 // dx = r*g - x * r^3 * mean(x*g), g = w*dy;   dw[c] += sum_rows dy*x*r   (fp32 atomics)
 // Optional `dres` is added to dx (fused residual-gradient add).
-template <int LPR, int MAXC>
-__global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
+template <int LPR, int MAXC, int THREADS>
+__global__ __launch_bounds__(THREADS) void rmsnorm_bwd_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ w, const bf16* __restrict__ dy,
     const bf16* __restrict__ dres, bf16* __restrict__ dx, float* __restrict__ dw, int64_t rows,
     int d, int64_t ldx, int64_t lddy, int64_t lddres, int64_t lddx, float eps) {
-  constexpr int RPB = 256 / LPR;
+  constexpr int RPB = THREADS / LPR;
   const int sub = threadIdx.x % LPR;
   const int rloc = threadIdx.x / LPR;
   float dwacc[MAXC][8];
@@ -151,18 +151,35 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(
       }
   }
   if (dw) {
-    // combine the RPB row-slots of this block in LDS, then one atomic per column per block
+    // Combine the RPB row-slots of this block in LDS, then one global atomic per column per
+    // block.  Global fp32 atomics are the expensive part (they are resolved beyond the per-XCD
+    // L2s, ~50 G/s), so the launch uses few, fat blocks; inside the block the slots add in turn
+    // (each lane owns its columns, so plain read-modify-write is enough).
     extern __shared__ float sdw[];  // d floats
-    for (int i = threadIdx.x; i < d; i += 256) sdw[i] = 0.f;
-    __syncthreads();
+#pragma unroll 1
+    for (int turn = 0; turn < RPB; turn++) {
+      if (rloc == turn) {
 #pragma unroll
-    for (int i = 0; i < MAXC; i++)
-      if ((i * LPR + sub) * 8 < d) {
+        for (int i = 0; i < MAXC; i++)
+          if ((i * LPR + sub) * 8 < d) {
+            float* dst = &sdw[(i * LPR + sub) * 8];
+            f32x4 lo, hi;
+            if (turn == 0) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) atomicAdd(&sdw[(i * LPR + sub) * 8 + e], dwacc[i][e]);
+              for (int e = 0; e < 4; e++) { lo[e] = dwacc[i][e]; hi[e] = dwacc[i][4 + e]; }
+            } else {
+              lo = *reinterpret_cast<f32x4*>(dst);
+              hi = *reinterpret_cast<f32x4*>(dst + 4);
+#pragma unroll
+              for (int e = 0; e < 4; e++) { lo[e] += dwacc[i][e]; hi[e] += dwacc[i][4 + e]; }
+            }
+            *reinterpret_cast<f32x4*>(dst) = lo;
+            *reinterpret_cast<f32x4*>(dst + 4) = hi;
+          }
       }
-    __syncthreads();
-    for (int i = threadIdx.x; i < d; i += 256) atomicAdd(&dw[i], sdw[i]);
+      __syncthreads();
+    }
+    for (int i = threadIdx.x; i < d; i += THREADS) atomicAdd(&dw[i], sdw[i]);
   }
 }
 
@@ -459,11 +476,11 @@ extern "C" int32_t olmax_rmsnorm_bwd(hipStream_t stream, const void* x, const vo
   bf16* dxp = (bf16*)dx;
   const size_t smem = dw ? (size_t)d * 4 : 0;
   if (vec && d % 8 == 0 && d <= 256) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<16, 2>), dim3(grid_for(rows, 16, 512)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<16, 2, 256>), dim3(grid_for(rows, 16, 256)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   } else if (vec && d % 8 == 0 && d <= 4096) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 8>), dim3(grid_for(rows, 4, 512)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 8, 512>), dim3(grid_for(rows, 8, 256)), dim3(512), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   } else if (vec && d % 8 == 0 && d <= 8192) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 16>), dim3(grid_for(rows, 4, 512)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 16, 256>), dim3(grid_for(rows, 4, 256)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   } else {
     hipLaunchKernelGGL(rmsnorm_bwd_generic, dim3(grid_for(rows, 1, 1 << 16)), dim3(256), 0, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   }
