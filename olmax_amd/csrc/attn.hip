@@ -176,7 +176,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
     bf16* __restrict__ O, float* __restrict__ LSE, int S, int H, int KH, int64_t ldq, int64_t ldk,
     int64_t ldv, int64_t ldo, float scale, int window, float cap) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [2][K 16K | V 16K]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform for the compiler too
   const int l32 = lane & 31, lhi = lane >> 5;
   const int nqt = (S + 127) >> 7;
   const WgCoord wg = decode_wg(blockIdx.x, (int)(gridDim.x / (nqt * (H / KH))), H / KH);
@@ -271,7 +272,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
 #pragma unroll
         for (int r = 0; r < 16; r++) mt = fmaxf(mt, st[jt][r]);
       if (!CAP) mt *= sc2;  // sc2 > 0: the max commutes with the scaling
-      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      mt = half_swap_max(mt);
       // Lazy rescaling: the running reference m only moves when some row's maximum grew by more
       // than 2^8; until then exp2(s - m) <= 256 stays well inside fp32/bf16 range and the
       // 64-register rescale of O is skipped (wave-uniform decision).
@@ -310,7 +311,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
     dma_wait_all();
     __syncthreads();
   }
-  const float ltot = lsum + __shfl_xor(lsum, 32, 64);
+  const float ltot = half_swap_sum(lsum);
   const float inv = ltot > 0.f ? 1.f / ltot : 0.f;
   if (qi < S) {
     bf16* op = O + ((int64_t)b * S + qi) * ldo + h * 128;
@@ -361,7 +362,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     bf16* __restrict__ dQ, int S, int H, int KH, int64_t ldq, int64_t ldk, int64_t ldv, int64_t lddo,
     int64_t lddq, float scale, int window, float cap) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform for the compiler too
   const int l32 = lane & 31, lhi = lane >> 5;
   const int nqt = (S + 127) >> 7;
   const WgCoord wg = decode_wg(blockIdx.x, (int)(gridDim.x / (nqt * (H / KH))), H / KH);
@@ -498,7 +500,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   constexpr int QT = 32;                   // query rows per iteration
   constexpr int STAGE = 2 * QT * 256 + 256;  // Q | dO | lse, delta
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform for the compiler too
   const int l32 = lane & 31, lhi = lane >> 5;
   // key tile 0 is seen by every query: rank order is already longest first
   const WgCoord wg = decode_wg(blockIdx.x, (int)(gridDim.x / ((S + 127) >> 7)), 1);

@@ -72,6 +72,17 @@ __device__ __forceinline__ unsigned lds_addr_of(const void* p) {
   return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)p;
 }
 
+// max / sum of a value with the one held by the lane 32 away (the other half of the wave),
+// through v_permlane32_swap: no trip through the LDS crossbar (ds_bpermute) and its latency.
+__device__ __forceinline__ float half_swap_max(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_swap_sum(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Wave64 all-reduce (sum) by xor shuffles.
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
