@@ -18,6 +18,7 @@
 // Backward is split in two deterministic kernels (no atomics): dK/dV with the key tile
 // stationary, dQ with the query tile stationary; each recomputes P from the saved LSE.
 #include "common.h"
+#include <type_traits>
 
 extern "C" int32_t olmax_fill_zero(hipStream_t stream, void* p, int64_t nbytes);
 
@@ -540,9 +541,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
   TileDma<QT> tq, tdo;
   tq.init(ldq, wv, lane);
   tdo.init(lddo, wv, lane);
-  auto load_tile = [&](int it, int stage) {
-    const int hq = kh * rep + it / ntile;
-    const int t = t_lo + it % ntile;
+  // (head, tile) of the next tile to load; heads of the K/V group outermost
+  int ld_h = kh * rep, ld_t = t_lo;
+  auto load_tile = [&](int stage) {
+    const int hq = ld_h, t = ld_t;
+    if (++ld_t > t_hi) {
+      ld_t = t_lo;
+      ++ld_h;
+    }
     if (t * QT + QT <= S) {
       tq.issue(Q + ((int64_t)b * S + t * QT) * ldq + hq * 128, lds0 + stage * STAGE, wv);
       tdo.issue(dO + ((int64_t)b * S + t * QT) * lddo + hq * 128, lds0 + stage * STAGE + QT * 256, wv);
@@ -553,31 +559,33 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
     if (tid < 2 * QT) {
       const int ii = min(t * QT + (tid & (QT - 1)), S - 1);
       const float* src = tid < QT ? LSE : DELTA;
-      sreg = src[((int64_t)b * H + hq) * S + ii];
-      if (tid < QT) sreg *= LOG2E;
+      sreg = src[((int64_t)b * H + hq) * S + ii];  // consumed by store_stats a whole iteration later
     }
   };
+  // (the log2 scaling of LSE happens here, not at the load: touching the loaded value there
+  // would make wave 0 wait out the memory latency at the top of every iteration)
   auto store_stats = [&](int stage) {
-    if (tid < 2 * QT) reinterpret_cast<float*>(smem + stage * STAGE + 2 * QT * 256)[tid] = sreg;
+    if (tid < 2 * QT) reinterpret_cast<float*>(smem + stage * STAGE + 2 * QT * 256)[tid] = tid < QT ? sreg * LOG2E : sreg;
   };
 
   FragAddr fa;
   fa.init(lane);
   const unsigned char* svt = smem + 2 * STAGE;  // [128 keys][128] V tile
   dma_tile<128>(V + (int64_t)b * S * ldv + kh * 128, ldv, j0, S, lds0 + 2 * STAGE, wv, lane);
-  load_tile(0, 0);
+  load_tile(0);
   store_stats(0);
   dma_wait_all();
   __syncthreads();
-  for (int it = 0; it < total; it++) {
-    const int cur = it & 1;
-    if (it + 1 < total) load_tile(it + 1, cur ^ 1);
-    const int t = t_lo + it % ntile;
+  // One iteration on the tile in stage CUR (a compile-time constant, so that every LDS address
+  // below is a loop-invariant register plus an immediate); `t` is the tile's query-tile index.
+  auto iteration = [&](auto cur_tag, int t, bool more) {
+    constexpr int CUR = decltype(cur_tag)::value;
+    if (more) load_tile(CUR ^ 1);
     const int ib = t * QT;  // first query of the tile
     // this wave sees the tile iff some i in [ib, ib+QT) has j <= i <= j + window for its keys
     const bool visible = (ib + QT - 1 >= jw0) && (window < 0 || ib <= jw0 + 31 + window);
     if (visible) {
-      const unsigned char* sq = smem + cur * STAGE;
+      const unsigned char* sq = smem + CUR * STAGE;
       const unsigned char* so = sq + QT * 256;
       const float* slse = reinterpret_cast<const float*>(sq + 2 * QT * 256);
       const float* sdel = slse + QT;
@@ -632,9 +640,20 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
           dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_tr(sq, u * 16, dt), dsb[u], dk[dt], 0, 0, 0);
         }
     }
-    if (it + 1 < total) store_stats(cur ^ 1);
+    if (more) store_stats(CUR ^ 1);
     dma_wait_all();
     __syncthreads();
+  };
+  {
+    int t = t_lo;  // query tile being consumed
+    for (int it = 0; it < total; it += 2) {
+      iteration(std::integral_constant<int, 0>(), t, it + 1 < total);
+      if (++t > t_hi) t = t_lo;
+      if (it + 1 < total) {
+        iteration(std::integral_constant<int, 1>(), t, it + 2 < total);
+        if (++t > t_hi) t = t_lo;
+      }
+    }
   }
   if (kj < S) {
     bf16* kp = dK + ((int64_t)b * S + kj) * lddk + kh * 128;
