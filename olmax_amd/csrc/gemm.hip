@@ -215,7 +215,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   //   * the steady state has no branches: past the end the DMA re-fetches the last k-tile and
   //     the reads fetch a stage nobody uses any more.
   constexpr int NM = TM * TN, NF = TM + TN;
-  static_assert(2 * NINS <= NM && 2 * NF <= NM, "not enough MFMA slots for the loads");
+  static_assert(2 * NINS <= NM && 2 * NF <= NM && NF + 1 <= NM && NINS + NF <= NM, "not enough MFMA slots for the loads");
   bf16x8 fa[2][TM], fb[2][TN];
   dma(0, 0, 0, NINS);
   if (KT > 1) {
@@ -244,25 +244,33 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
     for (int m = 0; m < NM; m++) {
       const int i = m / TN, j = m % TN;
       acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
-      if (m < TN) fb[1][m] = load_b1(sb, 1, m);
-      else if (m < NF) fa[1][m - TN] = load_a1(sa, 1, m - TN);
+      // (no read in slot 0: hoisted above the first MFMA it would make that MFMA's operand
+      // wait, an in-order counter, cover the new read's latency as well)
+      if (m >= 1 && m <= TN) fb[1][m - 1] = load_b1(sb, 1, m - 1);
+      else if (m > TN && m <= NF) fa[1][m - 1 - TN] = load_a1(sa, 1, m - 1 - TN);
       __builtin_amdgcn_sched_barrier(0);
     }
     // k-tile kt+1 has landed (issued one k-tile ago); every wave is done reading k-tile kt
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    // k-step 1 from registers; even slots issue the DMA of k-tile kt+2 into the retired stage,
-    // odd slots fetch k-step 0 of k-tile kt+1
+    // k-step 1 from registers; the slots issue the DMA of k-tile kt+2 into the retired stage and
+    // fetch k-step 0 of k-tile kt+1
 #pragma unroll
     for (int m = 0; m < NM; m++) {
       const int i = m / TN, j = m % TN;
       acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
-      if ((m & 1) == 0 && (m >> 1) < NINS) {
-        const int q = m >> 1;
+      // item k of the slot list: DMA issues and fragment reads alternate while both last; the
+      // list starts in slot 1 when it fits, so that the first MFMA goes out right behind the barrier
+      constexpr int FIRST = (NINS + NF <= NM - 1) ? 1 : 0;
+      constexpr int BOTH = NINS < NF ? NINS : NF;
+      const int k = m - FIRST;
+      int q = -1, f = -1;  // DMA instruction / fragment of this slot
+      if (k >= 0 && k < 2 * BOTH) { if (k & 1) f = k >> 1; else q = k >> 1; }
+      else if (k >= 2 * BOTH && k < NINS + NF) { if (NINS > NF) q = k - BOTH; else f = k - BOTH; }
+      if (q >= 0) {
         if (q < A_INS) dma16_s(ap, a_off[q], da + (q * NW + wave) * 1024);
         else dma16_s(bp, b_off[q - A_INS], db + ((q - A_INS) * NW + wave) * 1024);
-      } else if ((m & 1) == 1 && (m >> 1) < NF) {
-        const int f = m >> 1;
+      } else if (f >= 0) {
         if (f < TN) fb[0][f] = load_b1(nb, 0, f);
         else fa[0][f - TN] = load_a1(na, 0, f - TN);
       }
