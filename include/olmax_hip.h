@@ -83,6 +83,16 @@ int32_t olmax_qk_rope_bwd(olmax_stream_t stream, const void* dy, void* dx, const
                           int64_t tokens, int32_t heads, int32_t head_dim, int32_t seq_len,
                           int64_t lddy, int64_t lddx, int64_t ldx, float eps);
 
+/* ---- Gated MLP input projection with the activation fused into the GEMM epilogue:
+ * GatedMLP.forward, src/olmax/nn/mlp.py:69-73 (gate_proj, up_proj, act(gate) * up in one call).
+ * W = [Wgate; Wup] ([2F, K], row stride ldw); act_out [M, F]; gu_out ([M, 2F], optional when
+ * M % 256 == 0 and F % 128 == 0 and K % 64 == 0, required as scratch otherwise) receives gate|up
+ * for the backward pass.  act: 0 = silu, 1 = tanh-approximated gelu.  Results equal
+ * olmax_gemm_bf16 followed by olmax_glu_fwd bit for bit. */
+int32_t olmax_gemm_glu_bf16(olmax_stream_t stream, const void* X, const void* W, void* gu_out, void* act_out,
+                            int32_t M, int32_t F, int32_t K, int64_t ldx, int64_t ldw, int64_t ldgu,
+                            int64_t ldact, int32_t act);
+
 /* ---- Gated MLP activation: GatedMLP.forward, src/olmax/nn/mlp.py:69-73:
  * out = act(gate) * up, act 0 = silu, 1 = tanh-approximated gelu (jax.nn.gelu default,
  * src/olmax/nn/transformer/layer.py:133). */

@@ -123,6 +123,14 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   return t;
 }
 
+// GLU activations (GatedMLP, reference src/olmax/nn/mlp.py:69-73): jax.nn.silu and the tanh
+// form of jax.nn.gelu; shared by the elementwise GLU kernels and the GEMM's fused epilogue.
+__device__ __forceinline__ float act_silu(float g) { return g / (1.f + __expf(-g)); }
+constexpr float GELU_C = 0.7978845608028654f;  // sqrt(2/pi)
+__device__ __forceinline__ float act_gelu(float g) {
+  return 0.5f * g * (1.f + tanhf(GELU_C * (g + 0.044715f * g * g * g)));
+}
+
 // elementwise.hip, library-internal: olmax_adamw_dscale with the grid size (workgroups) exposed.
 int olmax_adamw_grid(hipStream_t stream, float* p, const void* g, float* m, float* v, void* shadow_bf16, int64_t n,
                      int32_t grad_is_bf16, float lr, float b1, float b2, float eps, float wd, int64_t step,

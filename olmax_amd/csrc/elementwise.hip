@@ -13,14 +13,9 @@
 
 namespace {
 
-__device__ __forceinline__ float act_silu(float g) { return g / (1.f + __expf(-g)); }
 __device__ __forceinline__ float act_silu_grad(float g) {
   const float s = 1.f / (1.f + __expf(-g));
   return s * (1.f + g * (1.f - s));
-}
-constexpr float GELU_C = 0.7978845608028654f;  // sqrt(2/pi)
-__device__ __forceinline__ float act_gelu(float g) {
-  return 0.5f * g * (1.f + tanhf(GELU_C * (g + 0.044715f * g * g * g)));
 }
 __device__ __forceinline__ float act_gelu_grad(float g) {
   const float t = tanhf(GELU_C * (g + 0.044715f * g * g * g));

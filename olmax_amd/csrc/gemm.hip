@@ -54,11 +54,17 @@ bool g_prof_on = false;
 std::vector<ProfRec> g_prof;
 std::mutex g_prof_mu;
 
-template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32>
+// GLU != 0 (1 silu, 2 tanh-gelu) turns the kernel into the fused gate/up projection of a gated
+// MLP: B is [Wgate; Wup] ([2F, K]), a block covers 128 features and loads their 128 gate rows
+// and 128 up rows, arranged in LDS so that every wave owns the gate AND the up columns of the
+// same 32 features; the epilogue writes act = f(gate) * up ([M, F], leading dimension ldr) and,
+// when Cv is given, gate|up ([M, 2F]) as the plain GEMM would.  N is F in that mode.
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32, int GLU = 0>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm_bf16_kernel(
     const bf16* __restrict__ A, const bf16* __restrict__ B, void* __restrict__ Cv,
     const bf16* __restrict__ R, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
     int64_t ldr, int tiles_m, int tiles_n) {
+  static_assert(GLU == 0 || (BN == 256 && WN == 64 && B_KC && !HAS_RES && !OUT_F32), "GLU epilogue: 256-wide NT tiles only");
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int TM = WM / 16, TN = WN / 16;  // accumulators of 16x16 per wave
   constexpr int WAVES_N = BN / WN;
@@ -90,7 +96,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   const int gm = min(tiles_m - first_m, GM);
   const int tile_m = first_m + (pid % group_sz) % gm;
   const int tile_n = (pid % group_sz) / gm;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int m0 = tile_m * BM, n0 = tile_n * (GLU ? BN / 2 : BN);  // GLU: first feature of the block
 
   // swizzles (see the bank-geometry note at the top of the file)
   auto kswz = [](int row) { return (row >> 1) & 7; };                         // [rows][64] tiles
@@ -118,7 +124,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
     const int p = (i * NW + wave) * 64 + lane;
     if (B_KC) {
       const int row = p >> 3, ph = p & 7;
-      b_off[i] = (unsigned)(((int64_t)row * ldb + ((ph ^ kswz(row)) << 3)) * 2);
+      // GLU: LDS row (wave w: 64w .. 64w+63) = gate rows of features 32w .. 32w+31, then their up rows
+      const int64_t grow = GLU ? (int64_t)((row >> 5) & 1) * N + (row >> 6) * 32 + (row & 31) : row;
+      b_off[i] = (unsigned)((grow * ldb + ((ph ^ kswz(row)) << 3)) * 2);
     } else {
       constexpr int CPR = BN / 8;
       const int kr = p / CPR, ph = p % CPR;
@@ -284,6 +292,30 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   dma_wait_all();  // the redundant tail DMAs must not outlive the workgroup's LDS allocation
 
   // ---- epilogue: accumulator lane -> column l16, rows 4*g16 + r of each 16x16 tile
+  if (GLU) {
+    bf16* act = const_cast<bf16*>(R);
+    bf16* gu = reinterpret_cast<bf16*>(Cv);
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int col = n0 + wn * 32 + j * 16 + l16;  // feature
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int64_t row = m0 + wm * WM + i * 16 + g16 * 4 + r;
+          // same roundings as the unfused path: gate and up are bf16 arrays, so is f(gate)
+          const bf16 gb = f2bf(acc[i][j][r]), ub = f2bf(acc[i][j + 2][r]);
+          const float gf = bf2f(gb);
+          const float a = bf2f(f2bf(GLU == 2 ? act_gelu(gf) : act_silu(gf)));
+          act[row * ldr + col] = f2bf(a * bf2f(ub));
+          if (gu) {
+            gu[row * ldc + col] = gb;
+            gu[row * ldc + N + col] = ub;
+          }
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -358,6 +390,36 @@ int launch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 2.0 * M * N * K;
     rec.key = (BM == 256 ? 256 : 128) | (A_KC << 12) | (B_KC << 13) | (HAS_RES << 14) | (OUT_F32 << 15);
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof.push_back(rec);
+  }
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+template <int GLU>
+int launch_glu(hipStream_t s, const bf16* A, const bf16* B, bf16* gu, bf16* act, int M, int F, int K, int64_t lda,
+               int64_t ldb, int64_t ldgu, int64_t ldact) {
+  constexpr int SMEM = 2 * (256 + 256) * BK * 2;
+  auto kern = gemm_bf16_kernel<256, 256, 128, 64, true, true, false, false, GLU>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+    attr_set = true;
+  }
+  const int tm = M / 256, tn = F / 128;
+  ProfRec rec{};
+  if (g_prof_on) {
+    (void)hipEventCreate(&rec.e0);
+    (void)hipEventCreate(&rec.e1);
+    (void)hipEventRecord(rec.e0, s);
+  }
+  hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(512), SMEM, s, A, B, (void*)gu, (const bf16*)act, M, F, K, lda, ldb,
+                     ldgu, ldact, tm, tn);
+  if (g_prof_on) {
+    (void)hipEventRecord(rec.e1, s);
+    rec.flops = 4.0 * M * F * K;
+    rec.key = 256 | (1 << 12) | (1 << 13) | (1 << 16);
     std::lock_guard<std::mutex> lk(g_prof_mu);
     g_prof.push_back(rec);
   }
@@ -507,4 +569,31 @@ extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void
   if (!a_kc && !b_kc) GO(false, false);
   GO(false, true);
 #undef GO
+}
+
+extern "C" int32_t olmax_glu_fwd(hipStream_t stream, const void* gate, const void* up, void* out, int64_t T, int32_t F,
+                                 int64_t ldg, int64_t ldu, int64_t ldo, int32_t act);
+
+// Gated-MLP input projection with the activation fused into the GEMM epilogue:
+// act_out[M, F] = f(X Wgate^T) * (X Wup^T), W = [Wgate; Wup] ([2F, K], row stride ldw); gu_out
+// ([M, 2F], optional) receives gate|up for the backward pass.  Falls back to the plain GEMM
+// plus olmax_glu_fwd (through a caller-provided gu_out) when the shape does not fit the tile.
+extern "C" int32_t olmax_gemm_glu_bf16(hipStream_t stream, const void* X, const void* W, void* gu_out, void* act_out,
+                                       int32_t M, int32_t F, int32_t K, int64_t ldx, int64_t ldw, int64_t ldgu,
+                                       int64_t ldact, int32_t act) {
+  OLMAX_CHECK(X && W && act_out, OLMAX_ERR_ARG, "olmax_gemm_glu_bf16: null operand");
+  OLMAX_CHECK(M > 0 && F > 0 && K > 0, OLMAX_ERR_SHAPE, "olmax_gemm_glu_bf16: M,F,K must be positive (got %d,%d,%d)", M, F, K);
+  OLMAX_CHECK(act == 0 || act == 1, OLMAX_ERR_ARG, "olmax_gemm_glu_bf16: act must be 0 (silu) or 1 (gelu-tanh)");
+  OLMAX_CHECK(ldx >= K && ldw >= K && ldact >= F && (!gu_out || ldgu >= 2 * (int64_t)F), OLMAX_ERR_SHAPE,
+              "olmax_gemm_glu_bf16: leading dimension smaller than row length");
+  const bool fits = aligned16(X) && aligned16(W) && ldx % 8 == 0 && ldw % 8 == 0 && K % BK == 0 && M % 256 == 0 &&
+                    F % 128 == 0 && (int64_t)(M / 256) * (F / 128) >= 128 && !g_force_tile;
+  if (fits) {
+    if (act == 0) return launch_glu<1>(stream, (const bf16*)X, (const bf16*)W, (bf16*)gu_out, (bf16*)act_out, M, F, K, ldx, ldw, ldgu, ldact);
+    return launch_glu<2>(stream, (const bf16*)X, (const bf16*)W, (bf16*)gu_out, (bf16*)act_out, M, F, K, ldx, ldw, ldgu, ldact);
+  }
+  OLMAX_CHECK(gu_out, OLMAX_ERR_ARG, "olmax_gemm_glu_bf16: this shape needs gu_out as scratch for the unfused path");
+  int rc = olmax_gemm_bf16(stream, X, W, gu_out, nullptr, M, 2 * F, K, ldx, ldw, ldgu, 0, 0, 0, 0);
+  if (rc) return rc;
+  return olmax_glu_fwd(stream, gu_out, (const bf16*)gu_out + F, act_out, M, F, ldgu, ldgu, ldact, act);
 }

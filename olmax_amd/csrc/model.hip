@@ -137,7 +137,7 @@ inline int hook_point(int point) { return g_hook.fn ? g_hook.fn(g_hook.ctx, poin
 
 int block_forward(hipStream_t s, const olmax_model_config* c, const olmax_block_weights* w, int window,
                   const float* cos_t, const float* sin_t, const bf16* x, bf16* y, const Acts& a,
-                  bool need_y = true) {
+                  bool need_y = true, bool save_gu = true) {
   const Dims m = dims_of(c);
   const int lt = c->layer_type;
   const float eps = c->eps;
@@ -175,8 +175,11 @@ int block_forward(hipStream_t s, const olmax_model_config* c, const olmax_block_
     RC(olmax_rmsnorm_fwd(s, a.h, lt == 0 ? w->mlp_norm : w->mlp_in_norm, a.hn, m.T, m.d, m.d, m.d, eps));
     mlp_in = a.hn;
   }
-  RC(lin_fwd(s, mlp_in, m.d, w->wgu, m.d, 2 * m.F, a.gu, 2 * m.F, nullptr, 0, m.T));
-  RC(olmax_glu_fwd(s, a.gu, a.gu + m.F, a.act, m.T, m.F, 2 * m.F, 2 * m.F, m.F, c->act));
+  // gate|up projection with the activation in the GEMM epilogue; gate|up themselves are only
+  // written when a backward pass will read them (a.gu doubles as scratch for odd shapes)
+  const bool fused_shape = m.T % 256 == 0 && m.F % 128 == 0 && m.d % 64 == 0 && (m.T / 256) * (m.F / 128) >= 128;
+  RC(olmax_gemm_glu_bf16(s, mlp_in, w->wgu, (save_gu || !fused_shape) ? a.gu : nullptr, a.act, (int)m.T, m.F, m.d, m.d,
+                         m.d, 2 * m.F, m.F, c->act));
   if (lt == 0) {
     if (need_y) RC(lin_fwd(s, a.act, m.F, w->wdown, m.F, m.d, y, m.d, a.h, m.d, m.T));
   } else {
@@ -417,7 +420,7 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
     Arena aa(w.acts_base + (keep ? (int64_t)l * w.acts_stride : 0));
     Acts acts = carve_acts(c, aa);
     RC(block_forward(s, c, &bw, windows[l], cos_tables[l], sin_tables[l], w.xs + (int64_t)l * Td,
-                     w.xs + (int64_t)(l + 1) * Td, acts));
+                     w.xs + (int64_t)(l + 1) * Td, acts, true, keep));
   }
   const bf16* xl = w.xs + (int64_t)nl * Td;
   RC(olmax_rmsnorm_fwd(s, xl, P + L.final_norm, w.hn, m.T, m.d, m.d, m.d, c->eps));

@@ -148,6 +148,26 @@ def glu_fwd(gate, up, act: str = "silu", out=None):
     return out
 
 
+def gated_mlp_in(x, w_gate_up, act: str = "silu", gate_up_out=None, save_gate_up: bool = True, out=None):
+    """GatedMLP.forward up to the down projection (reference src/olmax/nn/mlp.py:69-73):
+    act(x Wgate^T) * (x Wup^T) with the activation fused into the GEMM epilogue.
+    w_gate_up = [Wgate; Wup] ([2F, d]).  Returns (act_out [T, F], gate|up [T, 2F] or None)."""
+    _need_gpu(x, w_gate_up)
+    x = _rows2d(x)
+    T, d = x.shape
+    F = w_gate_up.shape[0] // 2
+    if out is None:
+        out = torch.empty(T, F, device=x.device, dtype=BF16)
+    fits = T % 256 == 0 and F % 128 == 0 and d % 64 == 0 and (T // 256) * (F // 128) >= 128
+    if gate_up_out is None and (save_gate_up or not fits):
+        gate_up_out = torch.empty(T, 2 * F, device=x.device, dtype=BF16)
+    check(_L().olmax_gemm_glu_bf16(stream_ptr(), ptr(x), ptr(w_gate_up), ptr(gate_up_out), ptr(out), i32(T), i32(F),
+                                   i32(d), i64(x.stride(0)), i64(w_gate_up.stride(0)),
+                                   i64(0 if gate_up_out is None else gate_up_out.stride(0)), i64(out.stride(0)),
+                                   i32(_ACT[act])))
+    return out, gate_up_out
+
+
 def glu_bwd(gate, up, dh, act: str = "silu", dgate=None, dup=None):
     _need_gpu(gate, up, dh)
     gate, up, dh = _rows2d(gate), _rows2d(up), _rows2d(dh)

@@ -175,6 +175,28 @@ def test_glu(act, T, F):
     check_close(dg, wg, "dgate"); check_close(du, wu, "dup")
 
 
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("T,F,d", [(2048, 2048, 256), (4096, 1024, 128), (96, 40, 24)])
+def test_gated_mlp_in_fused_epilogue(act, T, F, d):
+    """The GEMM with the GLU epilogue must equal GEMM + glu_fwd bit for bit (same tile, same
+    roundings), match the oracle, and not need the gate|up output on fused shapes."""
+    ops = _ops()
+    say(f"gated_mlp_in {act} T{T} F{F} d{d}")
+    x = bfr(T, d, seed=1); w = bfr(2 * F, d, seed=2, scale=d ** -0.5)
+    xc, wc = x.cuda(), w.cuda()
+    gu_plain = ops.gemm(xc, wc)
+    act_plain = ops.glu_fwd(gu_plain[:, :F], gu_plain[:, F:], act)
+    act_fused, gu_fused = ops.gated_mlp_in(xc, wc, act)
+    assert torch.equal(gu_fused, gu_plain) and torch.equal(act_fused, act_plain)
+    fits = T % 256 == 0 and F % 128 == 0 and d % 64 == 0 and (T // 256) * (F // 128) >= 128
+    act_only, none = ops.gated_mlp_in(xc, wc, act, save_gate_up=False)
+    assert torch.equal(act_only, act_plain) and ((none is None) == fits)
+    if T * F * d <= 2 ** 31:
+        gu_want = ref.linear_fwd(x.double(), w.double(), rt)
+        want = ref.glu_fwd(gu_want[:, :F], gu_want[:, F:], act, rt)
+        assert maxrel(act_fused, want) < 2e-2
+
+
 ATTN_CASES = [
     # B, S, H, KH, D, window, softcap
     (2, 256, 4, 4, 128, None, 0.0),
