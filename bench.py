@@ -19,12 +19,16 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16 = 2.5e15  # dense MFMA bf16 FLOP/s of one MI355X
-# HBM-side bytes per launch of the dominant kernel (fetch + write, averaged over its 129 launches
-# per step), from the two rocprofv3 --pmc runs summarised in
+# HBM-side bytes per launch (fetch + write) of the GEMM instantiations, averaged over each one's
+# launches in the 32-layer step, from the two rocprofv3 --pmc runs summarised in
 # profiles/gemm_traffic_pmc_llama7b_shapes.txt (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after
-# calibration against kernels of known size).
-GEMM_NT_TRAFFIC_BYTES = 2.06e9
-GEMM_NT_ALGORITHMIC_BYTES = 481 * 2 ** 20
+# calibration against a kernel of known size).  Keyed like olmax_gemm_profile_end.
+GEMM_TRAFFIC_BYTES = {
+    256: 1.404e9,                                   # A_MC,B_NC (dW)
+    256 | 1 << 12 | 1 << 13: 1.566e9,               # A_KC,B_KC (qkv, LM head)
+    256 | 1 << 12 | 1 << 13 | 1 << 14: 0.767e9,     # A_KC,B_KC + residual (o, down)
+    256 | 1 << 12 | 1 << 13 | 1 << 16: 2.586e9,     # A_KC,B_KC + GLU epilogue (gate+up)
+}
 
 
 def cpu_baseline(sample_tokens: int = 512):
@@ -125,14 +129,17 @@ def main():
     trainer.process_microbatch(*batches[0])
     torch.cuda.synchronize()
     cap = 64
-    keys = (ctypes.c_int32 * cap)(); ms = (ctypes.c_double * cap)(); fl = (ctypes.c_double * cap)(); ln = (ctypes.c_int64 * cap)()
-    n = L.olmax_gemm_profile_end(keys, ms, fl, ln, cap)
+    keys = (ctypes.c_int32 * cap)(); ms = (ctypes.c_double * cap)(); fl = (ctypes.c_double * cap)()
+    by = (ctypes.c_double * cap)(); ln = (ctypes.c_int64 * cap)()
+    n = L.olmax_gemm_profile_end(keys, ms, fl, by, ln, cap)
     per = []
     for i in range(n):
         k = keys[i]
-        name = "gemm_bf16_kernel<tile%d,%s,%s%s%s>" % (k & 0xfff, "A_KC" if k >> 12 & 1 else "A_MC", "B_KC" if k >> 13 & 1 else "B_NC",
-                                                       ",res" if k >> 14 & 1 else "", ",f32out" if k >> 15 & 1 else "")
-        per.append({"kernel": name, "launches": ln[i], "total_ms": ms[i], "avg_ms": ms[i] / ln[i], "tflops": fl[i] / ms[i] / 1e9})
+        name = "gemm_bf16_kernel<tile%d,%s,%s%s%s%s>" % (k & 0xfff, "A_KC" if k >> 12 & 1 else "A_MC", "B_KC" if k >> 13 & 1 else "B_NC",
+                                                         ",res" if k >> 14 & 1 else "", ",f32out" if k >> 15 & 1 else "",
+                                                         ",glu" if k >> 16 & 1 else "")
+        per.append({"kernel": name, "key": k, "launches": ln[i], "total_ms": ms[i], "avg_ms": ms[i] / ln[i],
+                    "tflops": fl[i] / ms[i] / 1e9, "algorithmic_bytes_per_launch": by[i] / ln[i]})
     per.sort(key=lambda r: -r["total_ms"])
     dom = per[0] if per else None
     gemm_ms = sum(r["total_ms"] for r in per)
@@ -141,8 +148,8 @@ def main():
     if dom:
         roofline = {"bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s",
                     "frac": dom["tflops"] / (PEAK_BF16 / 1e12),
-                    "traffic": GEMM_NT_TRAFFIC_BYTES if dom["kernel"].endswith("A_KC,B_KC>") and cfg.num_layers == 32 else None,
-                    "algorithmic_bytes": GEMM_NT_ALGORITHMIC_BYTES, "kernel": dom["kernel"],
+                    "traffic": GEMM_TRAFFIC_BYTES.get(dom["key"]) if cfg.num_layers == 32 else None,
+                    "algorithmic_bytes": dom["algorithmic_bytes_per_launch"], "kernel": dom["kernel"],
                     "avg_launch_ms": dom["avg_ms"], "launches_per_step": dom["launches"],
                     "all_gemm": {"ms_per_step": gemm_ms, "tflops": gemm_fl / gemm_ms if gemm_ms else None,
                                  "share_of_step": gemm_ms / ms_per_step}}

@@ -50,9 +50,12 @@ void olmax_gemm_set_tile(int tile);
 /* Diagnostic: record a HIP-event pair on the launch stream around every MFMA GEMM launch
  * between begin and end (allocates events; not for graph capture).  end() waits for them and
  * aggregates per kernel instantiation: key = tile | a_kc<<12 | b_kc<<13 | has_res<<14 |
- * out_f32<<15.  Returns the number of distinct keys written (at most cap). */
+ * out_f32<<15 | glu_epilogue<<16; ms = summed durations, flops / bytes = summed algorithmic
+ * work (2MNK; operands and result moved once).  Returns the number of distinct keys written
+ * (at most cap). */
 void olmax_gemm_profile_begin(void);
-int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, int64_t* launches, int32_t cap);
+int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, double* bytes, int64_t* launches,
+                               int32_t cap);
 
 /* ---- RMSNorm: rms_norm, src/olmax/nn/functional.py:51-67; RMSNorm.forward,
  * src/olmax/nn/normalization.py:85-87.  w may be NULL (no scale). */

@@ -48,6 +48,7 @@ constexpr int BK = 64;
 struct ProfRec {
   hipEvent_t e0, e1;
   double flops;
+  double bytes;  // algorithmic: every operand and the result moved once
   int key;  // tile | a_kc<<12 | b_kc<<13 | has_res<<14 | out_f32<<15
 };
 bool g_prof_on = false;
@@ -389,6 +390,7 @@ int launch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16
   if (g_prof_on) {
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 2.0 * M * N * K;
+    rec.bytes = 2.0 * ((double)M * K + (double)N * K + (double)M * N * (HAS_RES ? 2 : 1) * (OUT_F32 ? 2 : 1));
     rec.key = (BM == 256 ? 256 : 128) | (A_KC << 12) | (B_KC << 13) | (HAS_RES << 14) | (OUT_F32 << 15);
     std::lock_guard<std::mutex> lk(g_prof_mu);
     g_prof.push_back(rec);
@@ -419,6 +421,7 @@ int launch_glu(hipStream_t s, const bf16* A, const bf16* B, bf16* gu, bf16* act,
   if (g_prof_on) {
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 4.0 * M * F * K;
+    rec.bytes = 2.0 * ((double)M * K + 2.0 * F * K + (double)M * F * (gu ? 3 : 1));
     rec.key = 256 | (1 << 12) | (1 << 13) | (1 << 16);
     std::lock_guard<std::mutex> lk(g_prof_mu);
     g_prof.push_back(rec);
@@ -451,9 +454,11 @@ extern "C" void olmax_gemm_profile_begin(void) {
 }
 // Stop recording, wait for the recorded events and aggregate per kernel instantiation.
 // keys/ms/flops/launches: host arrays of `cap` entries; returns the number of distinct keys.
-// key = tile | a_layout<<12 | b_layout<<13 | has_residual<<14 | out_f32<<15, with a_layout /
-// b_layout bit SET when the operand is reduction-contiguous.
-extern "C" int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, int64_t* launches, int32_t cap) {
+// key = tile | a_layout<<12 | b_layout<<13 | has_residual<<14 | out_f32<<15 | glu_epilogue<<16,
+// with a_layout / b_layout bit SET when the operand is reduction-contiguous.  flops / bytes:
+// algorithmic totals (2MNK; every operand and the result moved once).
+extern "C" int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, double* bytes, int64_t* launches,
+                                          int32_t cap) {
   std::lock_guard<std::mutex> lk(g_prof_mu);
   g_prof_on = false;
   int n = 0;
@@ -466,10 +471,10 @@ extern "C" int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flo
       if (keys[i] == r.key) break;
     if (i == n) {
       if (n >= cap) continue;
-      keys[n] = r.key; ms[n] = 0; flops[n] = 0; launches[n] = 0;
+      keys[n] = r.key; ms[n] = 0; flops[n] = 0; bytes[n] = 0; launches[n] = 0;
       n++;
     }
-    ms[i] += t; flops[i] += r.flops; launches[i] += 1;
+    ms[i] += t; flops[i] += r.flops; bytes[i] += r.bytes; launches[i] += 1;
     (void)hipEventDestroy(r.e0);
     (void)hipEventDestroy(r.e1);
   }
