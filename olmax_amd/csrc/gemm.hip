@@ -64,7 +64,7 @@ template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bo
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm_bf16_kernel(
     const bf16* __restrict__ A, const bf16* __restrict__ B, void* __restrict__ Cv,
     const bf16* __restrict__ R, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-    int64_t ldr, int tiles_m, int tiles_n) {
+    int64_t ldr, int tiles_m, int tiles_n, int c_vec) {
   static_assert(GLU == 0 || (BN == 256 && WN == 64 && B_KC && !HAS_RES && !OUT_F32), "GLU epilogue: 256-wide NT tiles only");
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int TM = WM / 16, TN = WN / 16;  // accumulators of 16x16 per wave
@@ -252,7 +252,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
 #pragma unroll
     for (int m = 0; m < NM; m++) {
       const int i = m / TN, j = m % TN;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
+      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[0][j], fa[0][i], acc[i][j], 0, 0, 0);
       // (no read in slot 0: hoisted above the first MFMA it would make that MFMA's operand
       // wait, an in-order counter, cover the new read's latency as well)
       if (m >= 1 && m <= TN) fb[1][m - 1] = load_b1(sb, 1, m - 1);
@@ -267,7 +267,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
 #pragma unroll
     for (int m = 0; m < NM; m++) {
       const int i = m / TN, j = m % TN;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
+      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
       // item k of the slot list: DMA issues and fragment reads alternate while both last; the
       // list starts in slot 1 when it fits, so that the first MFMA goes out right behind the barrier
       constexpr int FIRST = (NINS + NF <= NM - 1) ? 1 : 0;
@@ -292,7 +292,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   }
   dma_wait_all();  // the redundant tail DMAs must not outlive the workgroup's LDS allocation
 
-  // ---- epilogue: accumulator lane -> column l16, rows 4*g16 + r of each 16x16 tile
+  // ---- epilogue.  The MFMAs ran with their operands swapped (B fragment as the instruction's A),
+  // so each accumulator is a transposed 16x16 tile: lane -> row l16, columns 4*g16 + r, i.e. four
+  // consecutive columns of one row of C per lane.
   if (GLU) {
     bf16* act = const_cast<bf16*>(R);
     bf16* gu = reinterpret_cast<bf16*>(Cv);
@@ -300,37 +302,89 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
     for (int i = 0; i < TM; i++)
 #pragma unroll
       for (int j = 0; j < 2; j++) {
-        const int col = n0 + wn * 32 + j * 16 + l16;  // feature
+        const int64_t row = m0 + wm * WM + i * 16 + l16;
+        const int col = n0 + wn * 32 + j * 16 + g16 * 4;  // first of this lane's 4 features
+        Pack4 pa, pg, pu;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const int64_t row = m0 + wm * WM + i * 16 + g16 * 4 + r;
           // same roundings as the unfused path: gate and up are bf16 arrays, so is f(gate)
-          const bf16 gb = f2bf(acc[i][j][r]), ub = f2bf(acc[i][j + 2][r]);
-          const float gf = bf2f(gb);
+          pg.e[r] = f2bf(acc[i][j][r]);
+          pu.e[r] = f2bf(acc[i][j + 2][r]);
+          const float gf = bf2f(pg.e[r]);
           const float a = bf2f(f2bf(GLU == 2 ? act_gelu(gf) : act_silu(gf)));
-          act[row * ldr + col] = f2bf(a * bf2f(ub));
+          pa.e[r] = f2bf(a * bf2f(pu.e[r]));
+        }
+        if (c_vec) {
+          *reinterpret_cast<u32x2*>(act + row * ldr + col) = pa.u;
           if (gu) {
-            gu[row * ldc + col] = gb;
-            gu[row * ldc + N + col] = ub;
+            *reinterpret_cast<u32x2*>(gu + row * ldc + col) = pg.u;
+            *reinterpret_cast<u32x2*>(gu + row * ldc + N + col) = pu.u;
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            act[row * ldr + col + r] = pa.e[r];
+            if (gu) {
+              gu[row * ldc + col + r] = pg.e[r];
+              gu[row * ldc + N + col + r] = pu.e[r];
+            }
           }
         }
       }
     return;
   }
+  if (!OUT_F32 && c_vec) {
+    // Through LDS (free now), so that C leaves in whole 128-byte lines: each wave parks its
+    // WM x 64 tile as bf16 rows of 128 B (16-byte chunks swizzled like the operand tiles), reads
+    // it back 16 B per lane -- 8 lanes per row -- and stores 8 full lines per instruction.  The
+    // residual is added in fp32 before the single rounding, as in the reference.
+    static_assert(WN == 64, "the staging layout assumes 64-column wave tiles");
+    __syncthreads();  // every wave is done reading the operand stages
+    unsigned char* ws = smem + wave * (WM * 128);
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int row = i * 16 + l16;
+        const int chunk = j * 2 + (g16 >> 1);
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] = acc[i][j][r];
+        if (HAS_RES) {
+          Pack4 rr;
+          rr.u = *reinterpret_cast<const u32x2*>(R + (int64_t)(m0 + wm * WM + row) * ldr + n0 + wn * WN + j * 16 + g16 * 4);
+#pragma unroll
+          for (int r = 0; r < 4; r++) v[r] += bf2f(rr.e[r]);
+        }
+        Pack4 pk;
+#pragma unroll
+        for (int r = 0; r < 4; r++) pk.e[r] = f2bf(v[r]);
+        *reinterpret_cast<u32x2*>(ws + row * 128 + ((chunk ^ kswz(row)) << 4) + ((g16 & 1) << 3)) = pk.u;
+      }
+    bf16* C = reinterpret_cast<bf16*>(Cv);
+#pragma unroll
+    for (int t = 0; t < WM / 8; t++) {
+      const int row = t * 8 + (lane >> 3), chunk = lane & 7;
+      const u32x4 line = *reinterpret_cast<const u32x4*>(ws + row * 128 + ((chunk ^ kswz(row)) << 4));
+      *reinterpret_cast<u32x4*>(C + (int64_t)(m0 + wm * WM + row) * ldc + n0 + wn * WN + chunk * 8) = line;
+    }
+    return;
+  }
+  // element-wise stores: fp32 output, or a C / R whose alignment rules out vector accesses
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      const int col = n0 + wn * WN + j * 16 + l16;
+      const int64_t row = m0 + wm * WM + i * 16 + l16;
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const int row = m0 + wm * WM + i * 16 + g16 * 4 + r;
+        const int col = n0 + wn * WN + j * 16 + g16 * 4 + r;
         float v = acc[i][j][r];
-        if (HAS_RES) v += bf2f(R[(int64_t)row * ldr + col]);
+        if (HAS_RES) v += bf2f(R[row * ldr + col]);
         if (OUT_F32)
-          reinterpret_cast<float*>(Cv)[(int64_t)row * ldc + col] = v;
+          reinterpret_cast<float*>(Cv)[row * ldc + col] = v;
         else
-          reinterpret_cast<bf16*>(Cv)[(int64_t)row * ldc + col] = f2bf(v);
+          reinterpret_cast<bf16*>(Cv)[row * ldc + col] = f2bf(v);
       }
     }
 }
@@ -385,8 +439,10 @@ int launch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16
     (void)hipEventCreate(&rec.e1);
     (void)hipEventRecord(rec.e0, s);
   }
+  // vector epilogue: 16-byte stores to C, 8-byte loads from R
+  const int c_vec = aligned16(C) && ldc % 8 == 0 && (!R || ((((uintptr_t)R) & 7) == 0 && ldr % 4 == 0));
   hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(NT), SMEM, s, A, B, C, R, M, N, K, lda, ldb, ldc,
-                     ldr, tm, tn);
+                     ldr, tm, tn, c_vec);
   if (g_prof_on) {
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 2.0 * M * N * K;
@@ -416,8 +472,9 @@ int launch_glu(hipStream_t s, const bf16* A, const bf16* B, bf16* gu, bf16* act,
     (void)hipEventCreate(&rec.e1);
     (void)hipEventRecord(rec.e0, s);
   }
+  const int c_vec = (((uintptr_t)act) & 7) == 0 && ldact % 4 == 0 && (!gu || ((((uintptr_t)gu) & 7) == 0 && ldgu % 4 == 0 && F % 4 == 0));
   hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(512), SMEM, s, A, B, (void*)gu, (const bf16*)act, M, F, K, lda, ldb,
-                     ldgu, ldact, tm, tn);
+                     ldgu, ldact, tm, tn, c_vec);
   if (g_prof_on) {
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 4.0 * M * F * K;
