@@ -142,6 +142,12 @@ int32_t olmax_lmhead_ce(olmax_stream_t stream, const void* h, const void* W, con
                         int64_t T, int32_t d, int32_t V, int32_t ignore_index, float softcap,
                         int32_t dw_f32);
 
+/* ---- Synthetic token batches: _randomize_start_offsets, src/olmax/data/utils.py:12-33:
+ * inputs[b, s] = (s + start_offsets[b]) mod V, targets = inputs + 1 (so a target equals V when
+ * the input is V - 1).  start_offsets: [B] int32 in [0, V-1), device memory, drawn by the caller. */
+int32_t olmax_sequential_tokens(olmax_stream_t stream, const int32_t* start_offsets, int32_t* inputs,
+                                int32_t* targets, int32_t B, int32_t S, int32_t V);
+
 /* ---- Embedding: Embedding.forward, src/olmax/nn/embedding.py:30-32 (row gather) and its
  * transpose (scatter-add; dW fp32 is ACCUMULATED into). */
 int32_t olmax_embed_fwd(olmax_stream_t stream, const int32_t* ids, const void* W, void* out, int64_t T,

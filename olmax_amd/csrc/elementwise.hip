@@ -98,6 +98,21 @@ __global__ void glu_bwd_scalar(const bf16* gate, const bf16* up, const bf16* dh,
   dup[t * lddu + c] = f2bf(df * (GELU ? act_gelu(gf) : act_silu(gf)));
 }
 
+// ------------------------------------------------------------------ synthetic token batches
+// inputs[b, s] = (s + offset[b]) mod V, targets = inputs + 1 (a target equals V, one past the
+// vocabulary, whenever the input is V - 1: the loss treats such a label as an all-zero one-hot).
+__global__ __launch_bounds__(256) void sequential_tokens_kernel(const int32_t* __restrict__ offsets,
+                                                                int32_t* __restrict__ inputs,
+                                                                int32_t* __restrict__ targets, int B, int S, int V) {
+  const int64_t total = (int64_t)B * S;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int b = (int)(i / S), sidx = (int)(i % S);
+    const int32_t tok = (int32_t)(((int64_t)sidx + offsets[b]) % V);
+    inputs[i] = tok;
+    targets[i] = tok + 1;
+  }
+}
+
 // ------------------------------------------------------------------ embedding
 // ids outside [0, V) are clamped (memory safety; the data path never produces them).
 __global__ __launch_bounds__(256) void embed_fwd_kernel(const int32_t* __restrict__ ids,
@@ -301,6 +316,17 @@ extern "C" int32_t olmax_embed_fwd(hipStream_t stream, const int32_t* ids, const
     hipLaunchKernelGGL(embed_fwd_kernel, dim3(grid_1d(T * (d / 8))), dim3(256), 0, stream, ids, (const bf16*)W, (bf16*)out, T, d, V);
   else
     hipLaunchKernelGGL(embed_fwd_scalar, dim3((unsigned)((T * d + 255) / 256)), dim3(256), 0, stream, ids, (const bf16*)W, (bf16*)out, T, d, V);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+extern "C" int32_t olmax_sequential_tokens(hipStream_t stream, const int32_t* start_offsets, int32_t* inputs,
+                                           int32_t* targets, int32_t B, int32_t S, int32_t V) {
+  if (B == 0 || S == 0) return OLMAX_OK;
+  OLMAX_CHECK(start_offsets && inputs && targets, OLMAX_ERR_ARG, "olmax_sequential_tokens: null pointer");
+  OLMAX_CHECK(B > 0 && S > 0 && V > 0, OLMAX_ERR_SHAPE, "olmax_sequential_tokens: bad shape");
+  hipLaunchKernelGGL(sequential_tokens_kernel, dim3(grid_1d((int64_t)B * S)), dim3(256), 0, stream, start_offsets, inputs,
+                     targets, B, S, V);
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
 }
