@@ -248,6 +248,22 @@ int32_t olmax_model_adamw(olmax_stream_t stream, const olmax_model_config* cfg, 
                           const float* grad_f32, int64_t step, float lr, float b1, float b2, float eps,
                           float wd, int32_t decay_embedding, float max_grad_norm, float* norm_scratch);
 
+/* Gradient accumulation over micro-batches: optax.MultiSteps as built at
+ * src/olmax/optim/config.py:153-154 and driven once per micro-batch by train_batch,
+ * src/olmax/train/trainer.py:779-807.  acc: fp32 [olmax_model_num_params], parameter layout;
+ * micro-batch mini_step (0-based) enters the running mean acc += (g - acc) / (mini_step + 1)
+ * (mini_step 0 overwrites).  olmax_grad_accumulate is the same for one flat array. */
+int32_t olmax_grad_accumulate(olmax_stream_t stream, float* acc, const void* g, int64_t n, int32_t grad_is_bf16,
+                              int32_t mini_step);
+int32_t olmax_model_grad_accumulate(olmax_stream_t stream, const olmax_model_config* cfg, float* acc,
+                                    const void* grad_bf16, const float* grad_f32, int32_t mini_step);
+/* AdamW (+ optional global-norm clip of the accumulated mean) from acc: the update MultiSteps
+ * applies on the last micro-batch of a batch. */
+int32_t olmax_model_adamw_accumulated(olmax_stream_t stream, const olmax_model_config* cfg, float* master,
+                                      float* m, float* v, void* params_bf16, const float* acc, int64_t step,
+                                      float lr, float b1, float b2, float eps, float wd,
+                                      int32_t decay_embedding, float max_grad_norm, float* norm_scratch);
+
 /* process_microbatch, src/olmax/train/trainer.py:759-777: loss + gradients + AdamW in one call.
  * opt_stream (optional, default priority, != stream): when given, clipping is off and the config
  * checkpoints its blocks, each layer's AdamW runs there concurrently with the recompute and

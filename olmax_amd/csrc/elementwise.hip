@@ -98,6 +98,44 @@ __global__ void glu_bwd_scalar(const bf16* gate, const bf16* up, const bf16* dh,
   dup[t * lddu + c] = f2bf(df * (GELU ? act_gelu(gf) : act_silu(gf)));
 }
 
+// ------------------------------------------------------------------ gradient accumulation
+// Running mean over micro-batches, acc += (g - acc) / (k + 1) for the k-th (0-based) micro-batch
+// (optax.MultiSteps with use_grad_mean, which the reference wraps its optimizer in,
+// src/olmax/optim/config.py:153-154); k = 0 overwrites acc.
+template <bool G_BF16>
+__global__ __launch_bounds__(256) void grad_accum_kernel(float* __restrict__ acc, const void* __restrict__ gv, int64_t n,
+                                                         float inv, int first) {
+  const int64_t n4 = n / 4;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+    float g[4];
+    if (G_BF16) {
+      Pack4 gp;
+      gp.u = reinterpret_cast<const u32x2*>(gv)[i];
+#pragma unroll
+      for (int e = 0; e < 4; e++) g[e] = bf2f(gp.e[e]);
+    } else {
+      const f32x4 gf = reinterpret_cast<const f32x4*>(gv)[i];
+#pragma unroll
+      for (int e = 0; e < 4; e++) g[e] = gf[e];
+    }
+    f32x4 a;
+    if (first) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) a[e] = g[e];
+    } else {
+      a = reinterpret_cast<const f32x4*>(acc)[i];
+#pragma unroll
+      for (int e = 0; e < 4; e++) a[e] = a[e] + (g[e] - a[e]) * inv;
+    }
+    reinterpret_cast<f32x4*>(acc)[i] = a;
+  }
+  if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    const int64_t i = n4 * 4 + threadIdx.x;
+    const float g = G_BF16 ? bf2f(reinterpret_cast<const bf16*>(gv)[i]) : reinterpret_cast<const float*>(gv)[i];
+    acc[i] = first ? g : acc[i] + (g - acc[i]) * inv;
+  }
+}
+
 // ------------------------------------------------------------------ synthetic token batches
 // inputs[b, s] = (s + offset[b]) mod V, targets = inputs + 1 (a target equals V, one past the
 // vocabulary, whenever the input is V - 1: the loss treats such a label as an all-zero one-hot).
@@ -316,6 +354,20 @@ extern "C" int32_t olmax_embed_fwd(hipStream_t stream, const int32_t* ids, const
     hipLaunchKernelGGL(embed_fwd_kernel, dim3(grid_1d(T * (d / 8))), dim3(256), 0, stream, ids, (const bf16*)W, (bf16*)out, T, d, V);
   else
     hipLaunchKernelGGL(embed_fwd_scalar, dim3((unsigned)((T * d + 255) / 256)), dim3(256), 0, stream, ids, (const bf16*)W, (bf16*)out, T, d, V);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+extern "C" int32_t olmax_grad_accumulate(hipStream_t stream, float* acc, const void* g, int64_t n, int32_t grad_is_bf16,
+                                         int32_t mini_step) {
+  if (n == 0) return OLMAX_OK;
+  OLMAX_CHECK(acc && g && n >= 0 && mini_step >= 0, OLMAX_ERR_ARG, "olmax_grad_accumulate: bad argument");
+  OLMAX_CHECK(aligned16(acc) && (((uintptr_t)g) & (grad_is_bf16 ? 7 : 15)) == 0, OLMAX_ERR_ALIGN,
+              "olmax_grad_accumulate: acc / fp32 g must be 16-byte aligned, bf16 g 8-byte aligned");
+  const int grid = grid_1d((n + 3) / 4, 2048);
+  const float inv = 1.f / (float)(mini_step + 1);
+  if (grad_is_bf16) hipLaunchKernelGGL(grad_accum_kernel<true>, dim3(grid), dim3(256), 0, stream, acc, g, n, inv, mini_step == 0);
+  else hipLaunchKernelGGL(grad_accum_kernel<false>, dim3(grid), dim3(256), 0, stream, acc, g, n, inv, mini_step == 0);
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
 }

@@ -708,6 +708,63 @@ extern "C" int32_t olmax_model_adamw(hipStream_t s, const olmax_model_config* c,
   return rc;
 }
 
+// Gradient accumulation over micro-batches (optax.MultiSteps, reference
+// src/olmax/optim/config.py:153-154): acc is an fp32 buffer in PARAMETER layout ([num_params]);
+// the k-th (0-based) micro-batch's gradients enter the running mean acc += (g - acc) / (k + 1).
+extern "C" int32_t olmax_model_grad_accumulate(hipStream_t s, const olmax_model_config* c, float* acc,
+                                               const void* grad_bf16, const float* grad_f32, int32_t mini_step) {
+  RC(check_cfg(c));
+  OLMAX_CHECK(acc && grad_bf16 && grad_f32 && mini_step >= 0, OLMAX_ERR_ARG, "olmax_model_grad_accumulate: bad argument");
+  const int nleaf = olmax_model_layout(c, nullptr, 0);
+  olmax_leaf* leaves = new olmax_leaf[nleaf];
+  olmax_model_layout(c, leaves, nleaf);
+  const bf16* G = (const bf16*)grad_bf16;
+  int rc = OLMAX_OK;
+  int i = 0;
+  while (i < nleaf && !rc) {
+    const olmax_leaf& lf = leaves[i];
+    if (lf.grad_f32) {
+      rc = olmax_grad_accumulate(s, acc + lf.offset, grad_f32 + lf.grad_f32_offset, lf.numel, 0, mini_step);
+      i++;
+    } else {  // runs of adjacent bf16-gradient leaves in one launch
+      int64_t n = lf.numel;
+      int j = i + 1;
+      while (j < nleaf && !leaves[j].grad_f32 && leaves[j].offset == lf.offset + n) n += leaves[j++].numel;
+      rc = olmax_grad_accumulate(s, acc + lf.offset, G + lf.offset, n, 1, mini_step);
+      i = j;
+    }
+  }
+  delete[] leaves;
+  return rc;
+}
+
+// AdamW from accumulated fp32 gradients in parameter layout (the step MultiSteps takes on its
+// last micro-batch); clipping (max_grad_norm > 0) acts on the accumulated mean, as the
+// reference chains it inside MultiSteps.
+extern "C" int32_t olmax_model_adamw_accumulated(hipStream_t s, const olmax_model_config* c, float* master, float* mom,
+                                                 float* var, void* params_bf16, const float* acc, int64_t step, float lr,
+                                                 float b1, float b2, float eps, float wd, int32_t decay_embedding,
+                                                 float max_grad_norm, float* norm_scratch) {
+  RC(check_cfg(c));
+  OLMAX_CHECK(master && mom && var && params_bf16 && acc, OLMAX_ERR_ARG, "olmax_model_adamw_accumulated: null pointer");
+  OLMAX_CHECK(step >= 1, OLMAX_ERR_ARG, "olmax_model_adamw_accumulated: step is 1-based");
+  OLMAX_CHECK(max_grad_norm <= 0.f || norm_scratch, OLMAX_ERR_ARG, "olmax_model_adamw_accumulated: clipping needs norm_scratch");
+  const Layout L = layout_of(c);
+  bf16* shadow = (bf16*)params_bf16;
+  const float* dscale = nullptr;
+  if (max_grad_norm > 0.f) {
+    RC(olmax_fill_zero(s, norm_scratch, 8));
+    RC(olmax_sumsq(s, acc, L.total, 0, norm_scratch));
+    hipLaunchKernelGGL(clip_scale_kernel, dim3(1), dim3(1), 0, s, norm_scratch, max_grad_norm, norm_scratch);
+    dscale = norm_scratch;
+  }
+  // the embedding (first in the layout) may be exempt from weight decay; everything else decays
+  const int64_t ne = L.layers_begin;
+  RC(olmax_adamw_dscale(s, master, acc, mom, var, shadow, ne, 0, lr, b1, b2, eps, decay_embedding ? wd : 0.f, step, 1.f, dscale));
+  return olmax_adamw_dscale(s, master + ne, acc + ne, mom + ne, var + ne, shadow + ne, L.total - ne, 0, lr, b1, b2, eps, wd,
+                            step, 1.f, dscale);
+}
+
 // One micro-batch of training: loss + gradients, then AdamW.  With a second stream and no
 // gradient clipping the optimizer update of each layer (HBM-bound) runs on `opt_stream`
 // concurrently with the backward pass of the layers below it (MFMA-bound); `stream` waits for

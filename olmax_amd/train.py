@@ -1,7 +1,7 @@
 """The train step of src/olmax/train/trainer.py:759-777 (process_microbatch) on the HIP path."""
 from __future__ import annotations
 
-from typing import Optional
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -26,6 +26,29 @@ class Trainer:
                                      eps=self.optim.eps, weight_decay=self.optim.weight_decay,
                                      decay_embedding=self._decay_embedding, max_grad_norm=self.optim.max_grad_norm,
                                      overlap_optimizer=self.overlap_optimizer)
+
+    def train_batch(self, batch: Sequence[Tuple[torch.Tensor, torch.Tensor]]) -> torch.Tensor:
+        """train_batch (reference src/olmax/train/trainer.py:779-807): one micro-batch at a time.
+        With one micro-batch this is process_microbatch.  With k > 1 the optimizer is wrapped in
+        optax.MultiSteps(k) (src/olmax/optim/config.py:153-154): each micro-batch's gradients
+        enter a running fp32 mean, the AdamW update (with the clip, on the mean) is applied after
+        the last one, and the schedule advances once per batch.  Returns the mean of the
+        micro-batch losses (trainer.py:796)."""
+        k = len(batch)
+        if k == 0:
+            raise ValueError("train_batch: empty batch")
+        if k == 1:
+            return self.process_microbatch(*batch[0])
+        lr = self.optim.lr_at(self.count)
+        self.count += 1
+        losses = []
+        for j, (ids, labels) in enumerate(batch):
+            losses.append(self.model.loss_and_grads(ids, labels).clone())
+            self.model.accumulate_grads(j)
+        self.model.adamw_step_accumulated(step=self.count, lr=lr, b1=self.optim.b1, b2=self.optim.b2, eps=self.optim.eps,
+                                          weight_decay=self.optim.weight_decay, decay_embedding=self._decay_embedding,
+                                          max_grad_norm=self.optim.max_grad_norm)
+        return torch.stack(losses).mean()
 
     @property
     def grad_norm(self) -> Optional[float]:

@@ -209,6 +209,7 @@ class Transformer:
         self.v: Optional[torch.Tensor] = None
         self.loss = torch.zeros((), device=dev, dtype=torch.float32)
         self.norm_scratch = torch.zeros(2, device=dev, dtype=torch.float32)
+        self.grad_acc = None  # fp32 running mean over micro-batches, allocated on first use
         self._workspace: Optional[torch.Tensor] = None
         self._opt_stream = None
 
@@ -321,6 +322,28 @@ class Transformer:
             ptr(self.grad_f32), ptr(ws), i64(ws.numel()), i64(step), f32(lr), f32(b1), f32(b2), f32(eps),
             f32(weight_decay), i32(int(decay_embedding)), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
         return self.loss
+
+    def accumulate_grads(self, mini_step: int) -> None:
+        """Fold the gradients of the micro-batch just differentiated into the running mean
+        ``self.grad_acc`` (fp32, parameter layout): optax.MultiSteps' accumulator, reference
+        src/olmax/optim/config.py:153-154.  ``mini_step`` is 0-based inside the batch."""
+        if self.grad_acc is None:
+            self.grad_acc = torch.zeros(self.num_params, device=self.device, dtype=torch.float32)
+        check(self._L.olmax_model_grad_accumulate(stream_ptr(), ctypes.byref(self.c), ptr(self.grad_acc),
+                                                  ptr(self.grad_bf16), ptr(self.grad_f32), i32(mini_step)))
+
+    def adamw_step_accumulated(self, *, step: int, lr: float, b1: float = 0.9, b2: float = 0.999, eps: float = 1e-8,
+                               weight_decay: float = 1e-4, decay_embedding: bool = True,
+                               max_grad_norm: Optional[float] = None) -> None:
+        """AdamW (and the optional global-norm clip) on the accumulated mean gradient."""
+        if self.m is None:
+            self.init_optimizer_state()
+        if self.grad_acc is None:
+            raise ValueError("adamw_step_accumulated: no gradients have been accumulated")
+        check(self._L.olmax_model_adamw_accumulated(
+            stream_ptr(), ctypes.byref(self.c), ptr(self.master), ptr(self.m), ptr(self.v), ptr(self.params_bf16),
+            ptr(self.grad_acc), i64(step), f32(lr), f32(b1), f32(b2), f32(eps), f32(weight_decay),
+            i32(int(decay_embedding)), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
 
     def init_optimizer_state(self) -> None:
         self.m = torch.zeros(self.num_params, device=self.device, dtype=torch.float32)

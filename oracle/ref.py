@@ -564,6 +564,38 @@ def train_step(cfg: ModelConfig, master: dict, opt: dict, ids, labels, *, step: 
     return loss, G
 
 
+def train_batch(cfg: ModelConfig, master: dict, opt: dict, batch, *, step: int, lr: float,
+                b1=0.9, b2=0.999, eps=1e-8, wd=1e-4, no_decay=("embedding.weight",),
+                compute_bf16: bool = False, max_grad_norm=None):
+    """train_batch (src/olmax/train/trainer.py:779-807) with the optimizer wrapped in
+    optax.MultiSteps(k) (src/olmax/optim/config.py:153-154; third party, restated from its
+    documentation: parity unpinned): gradients are cast to fp32 (trainer.py:738), the k
+    micro-batches enter the running mean acc += (g - acc) / (j + 1), the clip
+    (src/olmax/optim/utils.py:22-38) and AdamW act once, on the mean, and the reported loss is the
+    mean of the micro-batch losses.  `batch` = [(ids, labels), ...]."""
+    if compute_bf16:
+        P = {k: bf16_round(v) for k, v in master.items()}
+        rt = bf16_round
+    else:
+        P, rt = master, _id
+    acc, losses = None, []
+    for j, (ids, labels) in enumerate(batch):
+        loss, G = model_loss_and_grads(cfg, P, ids, labels, rt)
+        losses.append(loss)
+        G = {n: g.to(torch.float32).to(master[n].dtype) for n, g in G.items()}
+        acc = G if acc is None else {n: acc[n] + (G[n] - acc[n]) / (j + 1) for n in acc}
+    if max_grad_norm is not None:
+        norm = torch.sqrt(sum((g.double() ** 2).sum() for g in acc.values()))
+        scale = max_grad_norm / max(max_grad_norm, float(norm))
+        acc = {n: g * scale for n, g in acc.items()}
+    for name in master:
+        decay = 0.0 if any(_fnmatch(name, pat) for pat in no_decay) else wd
+        master[name], opt["m"][name], opt["v"][name] = adamw_step(
+            master[name], acc[name], opt["m"][name], opt["v"][name],
+            step=step, lr=lr, b1=b1, b2=b2, eps=eps, wd=decay)
+    return sum(losses) / len(losses), acc
+
+
 def _fnmatch(name: str, pat: str) -> bool:
     import fnmatch
 

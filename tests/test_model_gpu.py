@@ -210,3 +210,75 @@ def test_overlapped_optimizer_equals_sequential():
     assert outs[0][0] == pytest.approx(outs[1][0], rel=1e-5)
     assert relerr(outs[1][1], outs[0][1]) < 1e-5
     assert (outs[0][2].float() - outs[1][2].float()).abs().max() <= 1e-2 * outs[0][2].float().abs().max()
+
+
+def test_train_batch_gradient_accumulation_follows_oracle_and_mean_identity():
+    """train_batch with k micro-batches (optax.MultiSteps semantics: running fp32 mean of the
+    gradients, one clipped AdamW step per batch, loss = mean of micro-batch losses) against the
+    oracle on the tiny Llama, plus two properties that need no oracle: k copies of one micro-batch
+    equal a single step on it, and the accumulator equals the plain mean of the gradients."""
+    say("train_batch / gradient accumulation")
+    from olmax_amd import AdamWConfig, ConstantSchedule, Trainer, TransformerRecipe
+    hcfg = TransformerRecipe.tiny_llama()
+    ocfg = ref.ModelConfig(vocab=4096, d_model=256, n_layers=4, n_heads=4, n_kv_heads=4, head_dim=64, hidden=1024,
+                           eps=1e-6, rope_theta=1e4)
+    B, S, K = 2, 256, 3
+    master = ref.init_params(ocfg, seed=0)
+    init = {k: v.clone() for k, v in master.items()}
+
+    def batch_of(step):
+        out = []
+        for j in range(K):
+            gen = torch.Generator().manual_seed(100 * step + j)
+            ids = torch.randint(0, 4096, (B, S), generator=gen, dtype=torch.int32)
+            labels = torch.randint(0, 4096, (B, S), generator=gen, dtype=torch.int32)
+            out.append((ids, labels))
+        return out
+
+    opt_cfg = AdamWConfig(lr=ConstantSchedule(3e-4), b1=0.9, b2=0.95, weight_decay=0.1, max_grad_norm=1.0)
+    model = hcfg.build(batch_size=B, sequence_length=S)
+    model.load_state_dict(master)
+    tr = Trainer(model, opt_cfg)
+    opt = {"m": {k: torch.zeros_like(v) for k, v in master.items()}, "v": {k: torch.zeros_like(v) for k, v in master.items()}}
+    for step in range(1, 4):
+        batch = batch_of(step)
+        got = tr.train_batch([(i.cuda().reshape(-1), l.cuda().reshape(-1)) for i, l in batch]).item()
+        want, acc = ref.train_batch(ocfg, master, opt, [(i, l.long()) for i, l in batch], step=step, lr=3e-4, b1=0.9, b2=0.95,
+                                    wd=0.1, no_decay=(), compute_bf16=True, max_grad_norm=1.0)
+        assert abs(got - float(want)) < 1e-2 * abs(float(want))
+        assert tr.count == step
+    for n, p in model.named_parameters().items():
+        assert relerr(p, master[n]) < 1e-2, n
+    # the accumulator of the last batch is the clipped mean in the oracle; compare directions
+    leaves = {model.leaf_name(l): l for l in model.leaves}
+    for n in ("layers.1.mlp.down_proj.weight", "embedding.weight", "layers.0.attention_norm.weight"):
+        l = leaves[n]
+        assert cosine(model.grad_acc[l.offset: l.offset + l.numel].view(acc[n].shape), acc[n]) >= 0.999, n
+
+    # mean identity: accumulate three different gradients, compare with their plain mean
+    model2 = hcfg.build(batch_size=B, sequence_length=S)
+    model2.load_state_dict(init)
+    gs = []
+    for j, (ids, labels) in enumerate(batch_of(9)):
+        model2.loss_and_grads(ids.cuda().reshape(-1), labels.cuda().reshape(-1))
+        model2.accumulate_grads(j)
+        gs.append(model2.grad_bf16.float().clone())
+    l = leaves["layers.2.attention.q_proj.weight"]
+    sl = slice(l.offset, l.offset + l.numel)
+    mean = (gs[0][sl] + gs[1][sl] + gs[2][sl]) / 3
+    assert (model2.grad_acc[sl] - mean).abs().max() <= 1e-6 * mean.abs().max() + 1e-12
+
+    # k copies of one micro-batch == one step on it (no clipping, so the paths differ only in
+    # where the bf16 gradient is widened)
+    one = batch_of(5)[0]
+    dev = (one[0].cuda().reshape(-1), one[1].cuda().reshape(-1))
+    res = []
+    for k in (1, 2):
+        m = hcfg.build(batch_size=B, sequence_length=S)
+        m.load_state_dict(init)
+        t = Trainer(m, AdamWConfig(lr=ConstantSchedule(3e-4), b1=0.9, b2=0.95, weight_decay=0.1), overlap_optimizer=False)
+        t.train_batch([dev] * k)
+        res.append(m.master.clone())
+    # (a first Adam step is ~lr*sign(g): gradients summed by atomics in another order may flip
+    # near-zero entries, worth at most lr = 3e-4 against parameters of scale 0.02-0.1)
+    assert relerr(res[1], res[0]) < 5e-3
