@@ -75,6 +75,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-keep-activations-leg", action="store_true", help="skip the extra measurement without recompute")
     ap.add_argument("--no-overlap", action="store_true", help="run AdamW after the backward pass instead of overlapping it on a second stream")
+    ap.add_argument("--profiler-ranges", action="store_true", help="emit roctx ranges per layer and phase (for rocprofv3 --marker-trace)")
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline metric)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -88,6 +89,8 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(1)
     L = _lib.load()
+    if args.profiler_ranges:
+        Trainer.set_profiler_ranges(True)
     B, S = 2, 4096
     cfg = TransformerRecipe.llama_like_7B_bench()
     cfg.num_layers = args.layers

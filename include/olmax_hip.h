@@ -142,6 +142,13 @@ int32_t olmax_lmhead_ce(olmax_stream_t stream, const void* h, const void* W, con
                         int64_t T, int32_t d, int32_t V, int32_t ignore_index, float softcap,
                         int32_t dw_f32);
 
+/* ---- Profiler ranges: the counterpart of the reference's jax.named_scope annotations and
+ * ProfilerCallback (src/olmax/train/callbacks/profiler.py:33-50).  on != 0: the whole-model entry
+ * points emit roctx ranges ("olmax.layers.<l>.forward" / ".backward", "olmax.lm_head_and_loss")
+ * on the calling host thread, visible to rocprofv3 --marker-trace.  Needs libroctx64.so at run
+ * time; returns an error (and stays off) without it. */
+int32_t olmax_set_profiler_ranges(int32_t on);
+
 /* ---- Synthetic token batches: _randomize_start_offsets, src/olmax/data/utils.py:12-33:
  * inputs[b, s] = (s + start_offsets[b]) mod V, targets = inputs + 1 (so a target equals V when
  * the input is V - 1).  start_offsets: [B] int32 in [0, V-1), device memory, drawn by the caller. */

@@ -123,6 +123,10 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   return t;
 }
 
+// api.hip: roctx ranges around phases of the whole-model entry points (no-ops unless switched on)
+void olmax_range_push(const char* fmt, ...);
+void olmax_range_pop(void);
+
 // GLU activations (GatedMLP, reference src/olmax/nn/mlp.py:69-73): jax.nn.silu and the tanh
 // form of jax.nn.gelu; shared by the elementwise GLU kernels and the GEMM's fused epilogue.
 __device__ __forceinline__ float act_silu(float g) { return g / (1.f + __expf(-g)); }

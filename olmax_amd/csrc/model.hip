@@ -411,8 +411,19 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
   const int nl = c->n_layers;
   const bool keep = bwd && !c->checkpoint;
 
+  // RAII scope: a failing RC() return still closes the range
+  struct Range {
+    bool open = true;
+    Range(const char* f, int l) { olmax_range_push(f, l); }
+    void end() {
+      if (open) olmax_range_pop();
+      open = false;
+    }
+    ~Range() { end(); }
+  };
   RC(olmax_embed_fwd(s, ids, P + L.embedding, w.xs, m.T, m.d, c->vocab));
   for (int l = 0; l < nl; l++) {
+    Range rg("olmax.layers.%d.forward", l);
     LayerOff o;
     layer_offsets(c, l, L, plp, plf, o);
     olmax_block_weights bw;
@@ -422,6 +433,7 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
     RC(block_forward(s, c, &bw, windows[l], cos_tables[l], sin_tables[l], w.xs + (int64_t)l * Td,
                      w.xs + (int64_t)(l + 1) * Td, acts, true, keep));
   }
+  Range rg_head("olmax.lm_head_and_loss", 0);
   const bf16* xl = w.xs + (int64_t)nl * Td;
   RC(olmax_rmsnorm_fwd(s, xl, P + L.final_norm, w.hn, m.T, m.d, m.d, m.d, c->eps));
   const bf16* Wout = c->tied ? P + L.embedding : P + L.lm_head;
@@ -442,9 +454,11 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
   RC(olmax_rmsnorm_bwd(s, xl, P + L.final_norm, w.da, nullptr, w.db, grad_f32 + L.f_final_norm, m.T, m.d, m.d, m.d, 0,
                        m.d, c->eps));
   RC(ready(-1));
+  rg_head.end();
   bf16* dcur = w.db;
   bf16* dnext = w.da;
   for (int l = nl - 1; l >= 0; l--) {
+    Range rg("olmax.layers.%d.backward", l);
     LayerOff o;
     layer_offsets(c, l, L, plp, plf, o);
     olmax_block_weights bw;

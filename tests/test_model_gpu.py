@@ -282,3 +282,52 @@ def test_train_batch_gradient_accumulation_follows_oracle_and_mean_identity():
     # (a first Adam step is ~lr*sign(g): gradients summed by atomics in another order may flip
     # near-zero entries, worth at most lr = 3e-4 against parameters of scale 0.02-0.1)
     assert relerr(res[1], res[0]) < 5e-3
+
+
+def test_checkpoint_round_trip_resumes_the_run(tmp_path):
+    """save_checkpoint / load_checkpoint (TrainState of src/olmax/train/trainer.py:45-53): a run
+    resumed from the file continues like the uninterrupted one, including the data loader
+    position: the first resumed loss is bit-identical (same parameters, deterministic forward),
+    later ones agree to the noise of the atomically summed norm / embedding gradients (which an
+    early Adam step, ~lr*sign(g), amplifies).  Profiler ranges are switched on for the run."""
+    say("checkpoint round trip")
+    from olmax_amd import AdamWConfig, Trainer, TransformerRecipe, WarmupCosineDecaySchedule, data
+    hcfg = TransformerRecipe.tiny_llama()
+    B, S = 2, 128
+    ocfg = ref.ModelConfig(vocab=4096, d_model=256, n_layers=4, n_heads=4, n_kv_heads=4, head_dim=64, hidden=1024,
+                           eps=1e-6, rope_theta=1e4)
+    P = ref.init_params(ocfg, seed=3)
+    sched = WarmupCosineDecaySchedule(2, 6, 1e-3, 1e-5, 1e-5)
+    kw = dict(vocab_size=4096, sequence_length=S, global_batch_size_instances=B, total_batches=6)
+
+    def fresh():
+        m = hcfg.build(batch_size=B, sequence_length=S)
+        m.load_state_dict(P)
+        return Trainer(m, AdamWConfig(lr=sched, weight_decay=0.1, max_grad_norm=1.0), overlap_optimizer=False)
+
+    Trainer.set_profiler_ranges(True)
+    try:
+        tr, dl = fresh(), data.DataLoader(11, **kw)
+        losses = []
+        path = str(tmp_path / "state.safetensors")
+        for i, batch in enumerate(dl):
+            losses.append(tr.train_batch([(x.reshape(-1), y.reshape(-1)) for x, y in batch]).item())
+            if i == 2:
+                tr.save_checkpoint(path, data_loader=dl, tokens_seen=3 * B * S)
+        final = tr.model.master.clone()
+
+        tr2, dl2 = fresh(), data.DataLoader(0, **kw)
+        meta = tr2.load_checkpoint(path, data_loader=dl2)
+        assert meta["step"] == 3 and meta["tokens_seen"] == 3 * B * S and tuple(meta["data_loader_state"]) == (11, 3, 0)
+        assert tr2.count == 3 and dl2.get_state() == (11, 3, 0)
+        resumed = [tr2.train_batch([(x.reshape(-1), y.reshape(-1)) for x, y in batch]).item() for batch in dl2]
+    finally:
+        Trainer.set_profiler_ranges(False)
+    assert len(resumed) == 3
+    assert resumed[0] == losses[3]
+    assert resumed == pytest.approx(losses[3:], rel=1e-3)
+    assert relerr(tr2.model.master, final) < 2e-2
+    with pytest.raises(ValueError):
+        small = TransformerRecipe.tiny_llama()
+        small.num_layers = 2
+        Trainer(small.build(batch_size=B, sequence_length=S), AdamWConfig(lr=sched)).load_checkpoint(path)
