@@ -152,6 +152,26 @@ class TransformerRecipe:
         return TransformerConfig(vocab_size=50_304, d_model=1024, hidden_size=2816, num_layers=16, n_heads=8)
 
     @staticmethod
+    def llama3_8B() -> TransformerConfig:
+        """recipes.py:126-165 (GQA 32/8 heads, theta 5e5, vocab 128256, hidden 14336)."""
+        return TransformerConfig(vocab_size=128_256, d_model=4096, hidden_size=14_336, num_layers=32, n_heads=32,
+                                 n_kv_heads=8, rope_theta=500_000.0)
+
+    @staticmethod
+    def llama3_70B() -> TransformerConfig:
+        """recipes.py:168-200 (d 8192, 80 layers, GQA 64/8, full-block AC).  Its fp32 master
+        parameters and Adam moments (70.6 B x 12 B) do not fit one 288 GB GPU: sizes only."""
+        return TransformerConfig(vocab_size=128_256, d_model=8192, hidden_size=28_672, num_layers=80, n_heads=64,
+                                 n_kv_heads=8, rope_theta=500_000.0, layer_ac_policy="nothing_saveable")
+
+    @staticmethod
+    def olmo2_32B() -> TransformerConfig:
+        """recipes.py:246-282 (reordered norm, head-wise QK-norm, GQA 40/8, full-block AC)."""
+        return TransformerConfig(vocab_size=100_278, d_model=5120, hidden_size=27_648, num_layers=64, n_heads=40,
+                                 n_kv_heads=8, layer_type="reordered_norm", qk_norm_headwise=True,
+                                 layer_ac_policy="nothing_saveable")
+
+    @staticmethod
     def olmo2_7B() -> TransformerConfig:
         return TransformerConfig(vocab_size=100_278, d_model=4096, hidden_size=11008, num_layers=32, n_heads=32,
                                  layer_type="reordered_norm", qk_norm_headwise=True)

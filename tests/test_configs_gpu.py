@@ -170,3 +170,25 @@ def test_config3_llama7b_full_model():
     emb = model.named_parameters()["embedding.weight"]
     ws_rows = model.workspace().view(torch.bfloat16)[: 4 * cfg.d_model].view(4, cfg.d_model)
     assert torch.equal(ws_rows, emb[ids[:4].long()].to(BF))
+
+
+@pytest.mark.parametrize("name", ["llama3_8B", "olmo2_32B"])
+def test_gqa_recipes_two_layer_slices_full_width(name):
+    """Two-layer slices of the reference's grouped-query recipes at their real widths
+    (src/olmax/nn/transformer/recipes.py:126-165 and :246-282): llama3-8B (32 query / 8 KV heads,
+    SwiGLU 14336, vocab 128256) and OLMo2-32B (40 / 8 heads, d 5120, reordered norm + QK-norm,
+    hidden 27648); causal-prefix parity against the oracle at seq 2048, micro-batch 2."""
+    say(f"{name}: 2-layer slice at full width")
+    from olmax_amd import TransformerRecipe
+    hcfg = getattr(TransformerRecipe, name)()
+    hcfg.num_layers = 2
+    hcfg.norm_eps = 1e-6
+    hcfg.layer_ac_policy = "nothing_saveable"
+    ocfg = ref.ModelConfig(vocab=hcfg.vocab_size, d_model=hcfg.d_model, n_layers=2, n_heads=hcfg.n_heads,
+                           n_kv_heads=hcfg.n_kv_heads, head_dim=128, hidden=hcfg.hidden_size,
+                           layer_type="reordered" if hcfg.layer_type == "reordered_norm" else "pre",
+                           qk_norm=bool(hcfg.qk_norm_headwise), eps=1e-6, rope_theta=hcfg.rope_theta)
+    model, loss = _model_prefix_check(hcfg, ocfg, 2, 2048, seed=21)
+    # unit-RMS hidden state times an N(0, 0.02) head: logits ~ N(0, d * 0.02^2), so the loss at
+    # init is ln V + variance / 2
+    assert abs(loss - (math.log(hcfg.vocab_size) + hcfg.d_model * 0.02 ** 2 / 2)) < 0.3
