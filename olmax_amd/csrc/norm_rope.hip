@@ -276,9 +276,11 @@ __global__ __launch_bounds__(256) void qk_rope_bwd_kernel(
     __syncthreads();
   }
   const int sub = threadIdx.x & 15;
-  const int64_t unit = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
-  const bool live = unit < tokens * heads;
-  if (live) {
+  // a thread always serves the same 8 head-dim columns: its weight-gradient partials stay in
+  // registers over the grid-stride loop (few blocks, so few global atomics on the 128 addresses)
+  float dwacc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const int64_t units = tokens * heads;
+  for (int64_t unit = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4); unit < units; unit += (int64_t)gridDim.x * 16) {
     const int64_t tok = unit / heads;
     const int h = (int)(unit % heads);
     const int pos = (int)(tok % seq_len);
@@ -320,7 +322,7 @@ __global__ __launch_bounds__(256) void qk_rope_bwd_kernel(
 #pragma unroll
       for (int e = 0; e < 8; e++) {
         o.e[e] = f2bf(r * gg[e] - xf[e] * coef);
-        atomicAdd(&sdw[sub * 8 + e], g[e] * xf[e] * r);
+        dwacc[e] += g[e] * xf[e] * r;
       }
     } else {
 #pragma unroll
@@ -329,6 +331,8 @@ __global__ __launch_bounds__(256) void qk_rope_bwd_kernel(
     *reinterpret_cast<u32x4*>(dx + tok * lddx + h * 128 + sub * 8) = o.u;
   }
   if (NORM) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) atomicAdd(&sdw[sub * 8 + e], dwacc[e]);
     __syncthreads();
     if (threadIdx.x < 128) atomicAdd(&dw[threadIdx.x], sdw[threadIdx.x]);
   }
@@ -447,6 +451,8 @@ extern "C" int32_t olmax_rmsnorm_fwd_res(hipStream_t stream, const void* x, cons
     hipLaunchKernelGGL((rmsnorm_fwd_kernel<16, 2>), dim3(grid_for(rows, 16, 1 << 20)), dim3(256), 0, stream, xp, wp, rp, yp, rows, d, ldx, ldres, ldy, eps);
   } else if (vec && d % 8 == 0 && d <= 4096) {
     hipLaunchKernelGGL((rmsnorm_fwd_kernel<64, 8>), dim3(grid_for(rows, 4, 1 << 20)), dim3(256), 0, stream, xp, wp, rp, yp, rows, d, ldx, ldres, ldy, eps);
+  } else if (vec && d % 8 == 0 && d <= 6144) {
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<64, 12>), dim3(grid_for(rows, 4, 1 << 20)), dim3(256), 0, stream, xp, wp, rp, yp, rows, d, ldx, ldres, ldy, eps);
   } else if (vec && d % 8 == 0 && d <= 8192) {
     hipLaunchKernelGGL((rmsnorm_fwd_kernel<64, 16>), dim3(grid_for(rows, 4, 1 << 20)), dim3(256), 0, stream, xp, wp, rp, yp, rows, d, ldx, ldres, ldy, eps);
   } else {
@@ -479,6 +485,8 @@ extern "C" int32_t olmax_rmsnorm_bwd(hipStream_t stream, const void* x, const vo
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<16, 2, 256>), dim3(grid_for(rows, 16, 256)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   } else if (vec && d % 8 == 0 && d <= 4096) {
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 8, 512>), dim3(grid_for(rows, 8, 256)), dim3(512), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+  } else if (vec && d % 8 == 0 && d <= 6144) {
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 12, 512>), dim3(grid_for(rows, 8, 256)), dim3(512), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   } else if (vec && d % 8 == 0 && d <= 8192) {
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 16, 256>), dim3(grid_for(rows, 4, 256)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   } else {
@@ -532,7 +540,7 @@ extern "C" int32_t olmax_qk_rope_bwd(hipStream_t stream, const void* dy, void* d
     const int64_t units = tokens * heads;
     dim3 grid((unsigned)((units + 15) / 16));
     if (w)
-      hipLaunchKernelGGL(qk_rope_bwd_kernel<true>, grid, dim3(256), 0, stream, dyp, dxp, (const bf16*)x, (const bf16*)w, dw, cos_t, sin_t, tokens, heads, seq_len, lddy, lddx, ldx, eps);
+      hipLaunchKernelGGL(qk_rope_bwd_kernel<true>, dim3(grid.x < 1024 ? grid.x : 1024), dim3(256), 0, stream, dyp, dxp, (const bf16*)x, (const bf16*)w, dw, cos_t, sin_t, tokens, heads, seq_len, lddy, lddx, ldx, eps);
     else
       hipLaunchKernelGGL(qk_rope_bwd_kernel<false>, grid, dim3(256), 0, stream, dyp, dxp, (const bf16*)nullptr, (const bf16*)nullptr, (float*)nullptr, cos_t, sin_t, tokens, heads, seq_len, lddy, lddx, ldx, eps);
   } else {
