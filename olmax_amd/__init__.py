@@ -6,3 +6,4 @@ All arithmetic lives in hand-written HIP kernels behind the C ABI of ``libolmax_
 from .optim import AdamWConfig, ConstantSchedule, WarmupCosineDecaySchedule, WarmupStableDecaySchedule  # noqa: F401
 from .transformer import Transformer, TransformerConfig, TransformerRecipe  # noqa: F401
 from .train import Trainer  # noqa: F401
+from . import data  # noqa: F401,E402
