@@ -32,8 +32,9 @@
 // every XCD one contiguous run of tiles; runs walk the tile grid in column groups so that
 // the A row-panels and B column-panels a single L2 sees are re-used.
 #include "common.h"
-#include <vector>
 #include <mutex>
+#include <type_traits>
+#include <vector>
 
 namespace {
 
@@ -76,7 +77,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   constexpr int NINS = A_INS + B_INS;
   constexpr int STAGE = A_BYTES + B_BYTES;
 
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [2 stages][A tile | B tile]
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [A stage 0 | A stage 1 | B stage 0 | B stage 1]
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -105,35 +106,39 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
 
   // ---- DMA sources: instruction i of this wave fills LDS block (i*NW + wave) of 1 KB, i.e.
   // 16-byte chunks p = block*64 + lane of the tile; the lane fetches whichever global chunk the
-  // swizzle places there.  A lane's byte offset inside the operand panel never changes; the
-  // k-tile only moves the wave-uniform base (SGPRs), so the loop spends no VALU on addresses.
-  unsigned a_off[A_INS], b_off[B_INS];
-#pragma unroll
-  for (int i = 0; i < A_INS; i++) {
-    const int p = (i * NW + wave) * 64 + lane;
+  // swizzle places there.  Consecutive instructions of a wave are a whole number of swizzle
+  // periods (16 rows) apart, so a lane's byte offset inside the operand panel is one VGPR for all
+  // of them; instruction and k-tile only move the wave-uniform base (SGPRs), and the loop spends
+  // no vector instruction and one register per operand on DMA addresses.
+  unsigned a_off, b_off;
+  constexpr int A_IROWS = A_KC ? NW * 8 : NW * 64 / (BM / 8);  // tile rows between two instructions
+  constexpr int B_IROWS = B_KC ? NW * 8 : NW * 64 / (BN / 8);
+  static_assert(A_IROWS % 16 == 0 && B_IROWS % 16 == 0, "instructions of a wave must share the swizzle");
+  static_assert(GLU == 0 || B_IROWS == 64, "GLU row mapping: one instruction per wave tile of 64 rows");
+  {
+    const int p = wave * 64 + lane;
     if (A_KC) {
       const int row = p >> 3, ph = p & 7;
-      a_off[i] = (unsigned)(((int64_t)row * lda + ((ph ^ kswz(row)) << 3)) * 2);
+      a_off = (unsigned)(((int64_t)row * lda + ((ph ^ kswz(row)) << 3)) * 2);
     } else {
       constexpr int CPR = BM / 8;  // chunks per k-row
       const int kr = p / CPR, ph = p % CPR;
-      a_off[i] = (unsigned)(((int64_t)kr * lda + ((ph ^ tswz(kr)) << 3)) * 2);
+      a_off = (unsigned)(((int64_t)kr * lda + ((ph ^ tswz(kr)) << 3)) * 2);
     }
-  }
-#pragma unroll
-  for (int i = 0; i < B_INS; i++) {
-    const int p = (i * NW + wave) * 64 + lane;
     if (B_KC) {
       const int row = p >> 3, ph = p & 7;
-      // GLU: LDS row (wave w: 64w .. 64w+63) = gate rows of features 32w .. 32w+31, then their up rows
-      const int64_t grow = GLU ? (int64_t)((row >> 5) & 1) * N + (row >> 6) * 32 + (row & 31) : row;
-      b_off[i] = (unsigned)((grow * ldb + ((ph ^ kswz(row)) << 3)) * 2);
+      // GLU: LDS row (wave w: 64w .. 64w+63) = gate rows of features 32w .. 32w+31, then their up
+      // rows; instruction i covers LDS rows 64i .. 64i+63, i.e. 32 features further on per step
+      const int64_t grow = GLU ? (int64_t)((row >> 5) & 1) * N + (row & 31) : row;
+      b_off = (unsigned)((grow * ldb + ((ph ^ kswz(row)) << 3)) * 2);
     } else {
       constexpr int CPR = BN / 8;
       const int kr = p / CPR, ph = p % CPR;
-      b_off[i] = (unsigned)(((int64_t)kr * ldb + ((ph ^ tswz(kr)) << 3)) * 2);
+      b_off = (unsigned)(((int64_t)kr * ldb + ((ph ^ tswz(kr)) << 3)) * 2);
     }
   }
+  const int64_t a_istep = (int64_t)A_IROWS * lda;  // elements between two instructions' sources
+  const int64_t b_istep = (int64_t)(GLU ? 32 : B_IROWS) * ldb;
   const bf16* a_panel = A_KC ? A + (int64_t)m0 * lda : A + m0;  // k-tile 0 of this block's rows
   const bf16* b_panel = B_KC ? B + (int64_t)n0 * ldb : B + n0;
   const int64_t a_step = A_KC ? (int64_t)BK : (int64_t)BK * lda;
@@ -151,16 +156,16 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   const unsigned lds_base = lds_addr_of(smem);
   // issue DMA instructions [lo, hi) of the combined A+B list of k-tile kt into `stage`
   auto dma = [&](int kt, int stage, int lo, int hi) {
-    const unsigned sa = lds_base + stage * STAGE;
-    const unsigned sb = sa + A_BYTES;
+    const unsigned sa = lds_base + stage * A_BYTES;
+    const unsigned sb = lds_base + 2 * A_BYTES + stage * B_BYTES;
 #pragma unroll
     for (int i = 0; i < NINS; i++) {
       if (i < lo || i >= hi) continue;
       if (i < A_INS) {
-        dma16_s(a_panel + (int64_t)kt * a_step, a_off[i], sa + (i * NW + wave) * 1024);
+        dma16_s(a_panel + (int64_t)kt * a_step + i * a_istep, a_off, sa + (i * NW + wave) * 1024);
       } else {
         const int j = i - A_INS;
-        dma16_s(b_panel + (int64_t)kt * b_step, b_off[j], sb + (j * NW + wave) * 1024);
+        dma16_s(b_panel + (int64_t)kt * b_step + j * b_istep, b_off, sb + (j * NW + wave) * 1024);
       }
     }
   };
@@ -171,44 +176,83 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   // board's power limit (less accumulator traffic per FLOP).
   const int l16 = lane & 15, g16 = lane >> 4;
 
-  // one operand fragment (16 rows x 32 k) of k-step kk (0 or 1) of a stage
-  auto load_a1 = [&](const unsigned char* sa, int kk, int i) -> bf16x8 {
+  // Per-lane LDS byte addresses of the operand fragments, computed once.  LDS holds the A tiles
+  // of both stages first, then the B tiles ([A0 | A1 | B0 | B1]), so that one base register
+  // reaches a fragment of either stage with an immediate below 64 KB: for k-contiguous tiles one
+  // base per k-step with stage and tile row (i*16 rows = i*2048 B) as immediate; for transposed
+  // tiles one base per tile row -- the XOR swizzle permutes the chunk differently in every lane
+  // -- with stage, k-step and half ((kk*32 + h*4) k-rows) as immediate.  The bases pass through
+  // an empty asm so that the compiler keeps exactly these registers instead of re-deriving (and
+  // spilling) one address per read; the loop then holds no address arithmetic at all.
+  // (Adding whole 16-row tiles leaves kswz, which looks at row bits 1-3, unchanged; adding
+  // multiples of 4 k-rows leaves tswz unchanged as long as bit 3 of the k-row comes from the
+  // lane, which it does: k-row = 32*kk + 8*(lane/16) + 4*h + lane%16/4.)
+  constexpr int NA_BASE = A_KC ? 2 : TM, NB_BASE = B_KC ? 2 : TN;
+  static_assert(A_BYTES + 36 * (BM > BN ? BM : BN) * 2 < 65536, "fragment immediates must fit 16 bits");
+  unsigned a_base[NA_BASE], b_base[NB_BASE];
+#pragma unroll
+  for (int x = 0; x < NA_BASE; x++) {
+    unsigned v;
+    if (A_KC) {  // x = k-step
+      const int row = wm * WM + l16;
+      v = row * 128 + (((x * 4 + g16) ^ kswz(row)) << 4);
+    } else {     // x = tile row i
+      const int col = wm * WM + x * 16 + ((l16 & 3) << 2);
+      const int kr = g16 * 8 + (l16 >> 2);
+      v = kr * (BM * 2) + (((col >> 3) ^ tswz(kr)) << 4) + ((col & 7) << 1);
+    }
+    v += lds_base;
+    asm volatile("" : "+v"(v));
+    a_base[x] = v;
+  }
+#pragma unroll
+  for (int x = 0; x < NB_BASE; x++) {
+    unsigned v;
+    if (B_KC) {
+      const int row = wn * WN + l16;
+      v = row * 128 + (((x * 4 + g16) ^ kswz(row)) << 4);
+    } else {
+      const int col = wn * WN + x * 16 + ((l16 & 3) << 2);
+      const int kr = g16 * 8 + (l16 >> 2);
+      v = kr * (BN * 2) + (((col >> 3) ^ tswz(kr)) << 4) + ((col & 7) << 1);
+    }
+    v += lds_base + 2 * A_BYTES;
+    asm volatile("" : "+v"(v));
+    b_base[x] = v;
+  }
+  auto lds_b128 = [](unsigned addr) -> bf16x8 {
+    return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((uintptr_t)addr);
+  };
+  auto lds_tr64 = [](unsigned addr) -> u32x2 {
+    s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(uintptr_t)addr);
+    return (u32x2&)t;
+  };
+  // one operand fragment (16 rows x 32 k) of k-step kk (0 or 1) of stage st (all compile-time)
+  auto load_a1 = [&](int st, int kk, int i) -> bf16x8 {
     if (A_KC) {
-      const int row = wm * WM + i * 16 + l16;
-      const int ch = kk * 4 + g16;
-      return *reinterpret_cast<const bf16x8*>(sa + row * 128 + ((ch ^ kswz(row)) << 4));
+      return lds_b128(a_base[kk] + st * A_BYTES + i * 2048);
     } else {
       // transposing read: the 16-lane group g16 fetches k-rows kk*32 + 8*g16 + {0..3, 4..7}
-      const int col = wm * WM + i * 16 + ((l16 & 3) << 2);
       Pack8 p;
 #pragma unroll
       for (int h = 0; h < 2; h++) {
-        const int kr = kk * 32 + g16 * 8 + h * 4 + (l16 >> 2);
-        const int off = kr * (BM * 2) + (((col >> 3) ^ tswz(kr)) << 4) + ((col & 7) << 1);
-        s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)(sa + off));
-        p.u[h * 2 + 0] = ((u32x2&)t)[0];
-        p.u[h * 2 + 1] = ((u32x2&)t)[1];
+        const u32x2 t = lds_tr64(a_base[i] + st * A_BYTES + (kk * 32 + h * 4) * (BM * 2));
+        p.u[h * 2 + 0] = t[0];
+        p.u[h * 2 + 1] = t[1];
       }
       return p.v;
     }
   };
-  auto load_b1 = [&](const unsigned char* sb, int kk, int j) -> bf16x8 {
+  auto load_b1 = [&](int st, int kk, int j) -> bf16x8 {
     if (B_KC) {
-      const int row = wn * WN + j * 16 + l16;
-      const int ch = kk * 4 + g16;
-      return *reinterpret_cast<const bf16x8*>(sb + row * 128 + ((ch ^ kswz(row)) << 4));
+      return lds_b128(b_base[kk] + st * B_BYTES + j * 2048);
     } else {
-      const int col = wn * WN + j * 16 + ((l16 & 3) << 2);
       Pack8 p;
 #pragma unroll
       for (int h = 0; h < 2; h++) {
-        const int kr = kk * 32 + g16 * 8 + h * 4 + (l16 >> 2);
-        const int off = kr * (BN * 2) + (((col >> 3) ^ tswz(kr)) << 4) + ((col & 7) << 1);
-        s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)(sb + off));
-        p.u[h * 2 + 0] = ((u32x2&)t)[0];
-        p.u[h * 2 + 1] = ((u32x2&)t)[1];
+        const u32x2 t = lds_tr64(b_base[j] + st * B_BYTES + (kk * 32 + h * 4) * (BN * 2));
+        p.u[h * 2 + 0] = t[0];
+        p.u[h * 2 + 1] = t[1];
       }
       return p.v;
     }
@@ -224,8 +268,15 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   //   * the steady state has no branches: past the end the DMA re-fetches the last k-tile and
   //     the reads fetch a stage nobody uses any more.
   constexpr int NM = TM * TN, NF = TM + TN;
-  static_assert(2 * NINS <= NM && 2 * NF <= NM && NF + 1 <= NM && NINS + NF <= NM, "not enough MFMA slots for the loads");
-  bf16x8 fa[2][TM], fb[2][TN];
+  // Register budget: B fragments are needed by every MFMA row of a half and are double-buffered;
+  // an A fragment dies after its row (i-major MFMA order), so the first ASB of them are
+  // single-buffered -- the next k-step's data is fetched into the same registers right behind the
+  // row's last MFMA, a whole half ahead of its first use.  The last TM - ASB rows stay
+  // double-buffered so that no fetch is issued within ~8 MFMAs of the barrier that waits for it.
+  constexpr int ASB = BM == 256 ? 6 : 0, ND = TM - ASB;
+  static_assert(2 * NINS <= NM && NF + 1 <= NM && NINS + NF <= NM, "not enough MFMA slots for the loads");
+  static_assert(ASB == 0 || (NM >= 2 * NINS + 2 && NM >= 4 * (TN + ND)), "slot layout of the single-buffered scheme");
+  bf16x8 fas[ASB > 0 ? ASB : 1], fad[2][ND], fb[2][TN];
   dma(0, 0, 0, NINS);
   if (KT > 1) {
     dma(1, 1, 0, NINS);
@@ -235,65 +286,86 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   }
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < TM; i++) fa[0][i] = load_a1(smem, 0, i);
+  for (int i = 0; i < TM; i++) {
+    if (i < ASB) fas[i] = load_a1(0, 0, i);
+    else fad[0][i - ASB] = load_a1(0, 0, i);
+  }
 #pragma unroll
-  for (int j = 0; j < TN; j++) fb[0][j] = load_b1(smem + A_BYTES, 0, j);
+  for (int j = 0; j < TN; j++) fb[0][j] = load_b1(0, 0, j);
   // running DMA bases: k-tile kt+2 while it exists, then they stop advancing
   const bf16* ap = a_panel + (int64_t)min(2, KT - 1) * a_step;
   const bf16* bp = b_panel + (int64_t)min(2, KT - 1) * b_step;
-  for (int kt = 0; kt < KT; kt++) {
-    const int cur = kt & 1;
-    const unsigned char* sa = smem + cur * STAGE;
-    const unsigned char* sb = sa + A_BYTES;
-    const unsigned char* na = smem + (cur ^ 1) * STAGE;
-    const unsigned char* nb = na + A_BYTES;
-    const unsigned da = lds_base + cur * STAGE, db = da + A_BYTES;
-    // k-step 0 from registers; the fragments of k-step 1 are fetched meanwhile
+  // One k-tile.  The stage is a compile-time constant (the loop below is unrolled by two), so
+  // every LDS address is a loop-invariant per-lane register plus an immediate: no address
+  // arithmetic is left in the loop, where each vector instruction costs MFMA issue time.
+  auto k_tile = [&](int kt, auto cur_tag) {
+    constexpr int cur = decltype(cur_tag)::value;
+    constexpr int nxt = cur ^ 1;
+    const unsigned da = lds_base + cur * A_BYTES, db = lds_base + 2 * A_BYTES + cur * B_BYTES;
+    // ---- first half: k-step 0 from registers; the fragments of k-step 1 are fetched meanwhile
+    // (no fetch in slot 0: hoisted above the first MFMA it would make that MFMA's operand wait,
+    // an in-order counter, cover the new read's latency as well)
 #pragma unroll
     for (int m = 0; m < NM; m++) {
       const int i = m / TN, j = m % TN;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[0][j], fa[0][i], acc[i][j], 0, 0, 0);
-      // (no read in slot 0: hoisted above the first MFMA it would make that MFMA's operand
-      // wait, an in-order counter, cover the new read's latency as well)
-      if (m >= 1 && m <= TN) fb[1][m - 1] = load_b1(sb, 1, m - 1);
-      else if (m > TN && m <= NF) fa[1][m - 1 - TN] = load_a1(sa, 1, m - 1 - TN);
+      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[0][j], i < ASB ? fas[i] : fad[0][i < ASB ? 0 : i - ASB], acc[i][j], 0, 0, 0);
+      if (m >= 1 && m <= TN) fb[1][m - 1] = load_b1(cur, 1, m - 1);
+      if (m > TN && m <= TN + ND) fad[1][m - TN - 1] = load_a1(cur, 1, ASB + m - TN - 1);
+      if (j == TN - 1 && i < ASB) fas[i] = load_a1(cur, 1, i);
       __builtin_amdgcn_sched_barrier(0);
     }
     // k-tile kt+1 has landed (issued one k-tile ago); every wave is done reading k-tile kt
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    // k-step 1 from registers; the slots issue the DMA of k-tile kt+2 into the retired stage and
-    // fetch k-step 0 of k-tile kt+1
+    // ---- second half: k-step 1 from registers; the slots issue the DMA of k-tile kt+2 into the
+    // retired stage and fetch k-step 0 of k-tile kt+1; the first MFMA goes out right behind the barrier
 #pragma unroll
     for (int m = 0; m < NM; m++) {
       const int i = m / TN, j = m % TN;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
-      // item k of the slot list: DMA issues and fragment reads alternate while both last; the
-      // list starts in slot 1 when it fits, so that the first MFMA goes out right behind the barrier
-      constexpr int FIRST = (NINS + NF <= NM - 1) ? 1 : 0;
-      constexpr int BOTH = NINS < NF ? NINS : NF;
-      const int k = m - FIRST;
-      int q = -1, f = -1;  // DMA instruction / fragment of this slot
-      if (k >= 0 && k < 2 * BOTH) { if (k & 1) f = k >> 1; else q = k >> 1; }
-      else if (k >= 2 * BOTH && k < NINS + NF) { if (NINS > NF) q = k - BOTH; else f = k - BOTH; }
-      if (q >= 0) {
-        if (q < A_INS) dma16_s(ap, a_off[q], da + (q * NW + wave) * 1024);
-        else dma16_s(bp, b_off[q - A_INS], db + ((q - A_INS) * NW + wave) * 1024);
-      } else if (f >= 0) {
-        if (f < TN) fb[0][f] = load_b1(nb, 0, f);
-        else fa[0][f - TN] = load_a1(na, 0, f - TN);
+      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[1][j], i < ASB ? fas[i] : fad[1][i < ASB ? 0 : i - ASB], acc[i][j], 0, 0, 0);
+      int q = -1, f = -1;  // DMA instruction / double-buffered fragment of this slot
+      if (ASB > 0) {
+        // even slots from 2: DMA; slots 1, 5, 9, ...: B then double-buffered A fragments
+        if (m >= 2 && (m & 1) == 0 && (m >> 1) - 1 < NINS) q = (m >> 1) - 1;
+        if ((m & 3) == 1 && (m >> 2) < TN + ND) f = m >> 2;
+      } else {
+        // DMA issues and fragment reads alternate while both last, from slot 1 when they fit
+        constexpr int FIRST = (NINS + NF <= NM - 1) ? 1 : 0;
+        constexpr int BOTH = NINS < NF ? NINS : NF;
+        const int k = m - FIRST;
+        if (k >= 0 && k < 2 * BOTH) { if (k & 1) f = k >> 1; else q = k >> 1; }
+        else if (k >= 2 * BOTH && k < NINS + NF) { if (NINS > NF) q = k - BOTH; else f = k - BOTH; }
       }
+      if (q >= 0) {
+        if (q < A_INS) dma16_s(ap + q * a_istep, a_off, da + (q * NW + wave) * 1024);
+        else dma16_s(bp + (q - A_INS) * b_istep, b_off, db + ((q - A_INS) * NW + wave) * 1024);
+      }
+      if (f >= 0) {
+        if (f < TN) fb[0][f] = load_b1(nxt, 0, f);
+        else fad[0][f - TN] = load_a1(nxt, 0, ASB + f - TN);
+      }
+      if (j == TN - 1 && i < ASB) fas[i] = load_a1(nxt, 0, i);
       __builtin_amdgcn_sched_barrier(0);
     }
     if (kt + 3 < KT) {
       ap += a_step;
       bp += b_step;
     }
+  };
+  for (int kt = 0; kt + 1 < KT; kt += 2) {
+    k_tile(kt, std::integral_constant<int, 0>());
+    k_tile(kt + 1, std::integral_constant<int, 1>());
   }
+  if (KT & 1) k_tile(KT - 1, std::integral_constant<int, 0>());
   dma_wait_all();  // the redundant tail DMAs must not outlive the workgroup's LDS allocation
+  // The epilogue derives its addresses from a copy of the lane id that the compiler cannot see
+  // through, so none of them is computed ahead of the loop and kept in registers across it.
+  int lane_e = lane;
+  asm volatile("" : "+v"(lane_e));
+  const int l16e = lane_e & 15, g16e = lane_e >> 4;
 
   // ---- epilogue.  The MFMAs ran with their operands swapped (B fragment as the instruction's A),
-  // so each accumulator is a transposed 16x16 tile: lane -> row l16, columns 4*g16 + r, i.e. four
+  // so each accumulator is a transposed 16x16 tile: lane -> row l16e, columns 4*g16e + r, i.e. four
   // consecutive columns of one row of C per lane.
   if (GLU) {
     bf16* act = const_cast<bf16*>(R);
@@ -302,8 +374,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
     for (int i = 0; i < TM; i++)
 #pragma unroll
       for (int j = 0; j < 2; j++) {
-        const int64_t row = m0 + wm * WM + i * 16 + l16;
-        const int col = n0 + wn * 32 + j * 16 + g16 * 4;  // first of this lane's 4 features
+        const int64_t row = m0 + wm * WM + i * 16 + l16e;
+        const int col = n0 + wn * 32 + j * 16 + g16e * 4;  // first of this lane's 4 features
         Pack4 pa, pg, pu;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -345,26 +417,26 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
     for (int i = 0; i < TM; i++)
 #pragma unroll
       for (int j = 0; j < TN; j++) {
-        const int row = i * 16 + l16;
-        const int chunk = j * 2 + (g16 >> 1);
+        const int row = i * 16 + l16e;
+        const int chunk = j * 2 + (g16e >> 1);
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) v[r] = acc[i][j][r];
         if (HAS_RES) {
           Pack4 rr;
-          rr.u = *reinterpret_cast<const u32x2*>(R + (int64_t)(m0 + wm * WM + row) * ldr + n0 + wn * WN + j * 16 + g16 * 4);
+          rr.u = *reinterpret_cast<const u32x2*>(R + (int64_t)(m0 + wm * WM + row) * ldr + n0 + wn * WN + j * 16 + g16e * 4);
 #pragma unroll
           for (int r = 0; r < 4; r++) v[r] += bf2f(rr.e[r]);
         }
         Pack4 pk;
 #pragma unroll
         for (int r = 0; r < 4; r++) pk.e[r] = f2bf(v[r]);
-        *reinterpret_cast<u32x2*>(ws + row * 128 + ((chunk ^ kswz(row)) << 4) + ((g16 & 1) << 3)) = pk.u;
+        *reinterpret_cast<u32x2*>(ws + row * 128 + ((chunk ^ kswz(row)) << 4) + ((g16e & 1) << 3)) = pk.u;
       }
     bf16* C = reinterpret_cast<bf16*>(Cv);
 #pragma unroll
     for (int t = 0; t < WM / 8; t++) {
-      const int row = t * 8 + (lane >> 3), chunk = lane & 7;
+      const int row = t * 8 + (lane_e >> 3), chunk = lane_e & 7;
       const u32x4 line = *reinterpret_cast<const u32x4*>(ws + row * 128 + ((chunk ^ kswz(row)) << 4));
       *reinterpret_cast<u32x4*>(C + (int64_t)(m0 + wm * WM + row) * ldc + n0 + wn * WN + chunk * 8) = line;
     }
@@ -375,10 +447,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   for (int i = 0; i < TM; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      const int64_t row = m0 + wm * WM + i * 16 + l16;
+      const int64_t row = m0 + wm * WM + i * 16 + l16e;
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const int col = n0 + wn * WN + j * 16 + g16 * 4 + r;
+        const int col = n0 + wn * WN + j * 16 + g16e * 4 + r;
         float v = acc[i][j][r];
         if (HAS_RES) v += bf2f(R[row * ldr + col]);
         if (OUT_F32)
