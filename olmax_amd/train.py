@@ -9,6 +9,72 @@ from .optim import AdamWConfig
 from .transformer import Transformer
 
 
+class RunningAverage:
+    """Online mean and variance (Welford), the statistic behind the reference's averaged
+    throughput metrics (src/olmax/utils.py:209-246)."""
+
+    def __init__(self) -> None:
+        self.reset()
+
+    def reset(self) -> None:
+        self.mean, self.m2, self.count = 0.0, 0.0, 0
+
+    def update(self, value: float) -> float:
+        self.count += 1
+        d = value - self.mean
+        self.mean += d / self.count
+        self.m2 += d * (value - self.mean)
+        return self.mean
+
+    def get(self) -> float:
+        if self.count == 0:
+            raise ZeroDivisionError("no samples")
+        return self.mean
+
+    def get_variance(self) -> float:
+        if self.count < 2:
+            raise ZeroDivisionError("variance needs two samples")
+        return self.m2 / self.count
+
+    def get_sample_variance(self) -> float:
+        if self.count < 2:
+            raise ZeroDivisionError("variance needs two samples")
+        return self.m2 / (self.count - 1)
+
+
+class ThroughputMeter:
+    """Batches and tokens per second as the reference reports them (src/olmax/train/trainer.py:596-627):
+    the instantaneous rate every step; the running average from the 10th step of a run on (the first
+    steps carry compilation and warm-up there); the sample standard deviation once the average holds
+    5 samples.  One GPU: the per-device figures equal the global ones."""
+
+    def __init__(self, n_devices: int = 1) -> None:
+        self.avg = RunningAverage()
+        self.n_devices = n_devices
+
+    def update(self, step_this_run: int, seconds: float, tokens_this_batch: Optional[int]) -> dict:
+        import math
+
+        bps = 1.0 / seconds
+        bps_avg = None if step_this_run < 10 else self.avg.update(bps)
+        bps_std = None if self.avg.count < 5 else math.sqrt(self.avg.get_sample_variance())
+        out = {"throughput/BPS": bps}
+        if bps_avg is not None:
+            out["throughput/BPS average"] = bps_avg
+        if bps_std is not None:
+            out["throughput/BPS stddev"] = bps_std
+        if tokens_this_batch is not None:
+            out["throughput/TPS"] = bps * tokens_this_batch
+            out["throughput/TPS device"] = out["throughput/TPS"] / self.n_devices
+            if bps_avg is not None:
+                out["throughput/TPS average"] = bps_avg * tokens_this_batch
+                out["throughput/TPS device average"] = out["throughput/TPS average"] / self.n_devices
+            if bps_std is not None:
+                out["throughput/TPS stddev"] = bps_std * tokens_this_batch
+                out["throughput/TPS device stddev"] = out["throughput/TPS stddev"] / self.n_devices
+        return out
+
+
 class Trainer:
     """Minimal step driver: loss + grads, then the fused AdamW update, once per micro-batch."""
 
@@ -49,6 +115,69 @@ class Trainer:
                                           weight_decay=self.optim.weight_decay, decay_embedding=self._decay_embedding,
                                           max_grad_norm=self.optim.max_grad_norm)
         return torch.stack(losses).mean()
+
+    # ------------------------------------------------------------------ metrics and the training loop
+    def record_metric(self, name: str, value) -> None:
+        """Queue a metric of the current step (reference record_metric, src/olmax/train/trainer.py:274-278).
+        A device scalar starts its copy to pinned host memory on the current stream and is only read
+        when the step is logged, one step later, so logging never drains the GPU queue."""
+        if not hasattr(self, "_metrics"):
+            self._metrics = {}
+        if isinstance(value, torch.Tensor) and value.is_cuda:
+            host = torch.empty((), dtype=value.dtype, pin_memory=True)
+            host.copy_(value.detach().reshape(()), non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+            value = (host, ev)
+        self._metrics.setdefault(self.count, {})[name] = value
+
+    def _log_metrics(self, log_fn, exclude: Optional[int] = None) -> None:
+        import math
+
+        for step in sorted(getattr(self, "_metrics", {})):
+            if step == exclude:
+                continue
+            out = {}
+            for name, v in self._metrics.pop(step).items():
+                if isinstance(v, tuple):
+                    v[1].synchronize()
+                    v = float(v[0])
+                out[name] = float(v)
+            if log_fn is not None:
+                log_fn(step, out)
+            loss = out.get("train/loss")
+            if loss is not None and not math.isfinite(loss):
+                raise RuntimeError(f"NaN loss encountered on step {step}!")
+
+    def fit(self, data_loader, max_steps: int, log_fn=None, tokens_per_batch: Optional[int] = None) -> None:
+        """The reference's training loop (src/olmax/train/trainer.py:531-637) on one GPU.  Every item
+        of `data_loader` is one batch, a list of (input_ids, labels) micro-batches as
+        data.DataLoader yields them.  Per step: train on the batch, queue train/loss, optim/lr and
+        (when clipping) optim/g_norm, hand the metrics of earlier steps to `log_fn(step, dict)`
+        while this step still runs on the GPU, and record batches and tokens per second."""
+        import time
+
+        meter = ThroughputMeter()
+        step_this_run = 0
+        t0 = time.perf_counter()
+        for batch in data_loader:
+            if self.count >= max_steps:
+                break
+            step_this_run += 1
+            tokens = tokens_per_batch if tokens_per_batch is not None else sum(int(ids.numel()) for ids, _ in batch)
+            lr = self.optim.lr_at(self.count)  # read before the count moves: the first step uses schedule(0)
+            loss = self.train_batch([(ids.reshape(-1), labels.reshape(-1)) for ids, labels in batch])
+            self.record_metric("train/loss", loss)
+            self.record_metric("optim/lr", lr)
+            if self.optim.max_grad_norm is not None:
+                self.record_metric("optim/g_norm", self.model.norm_scratch[1])
+            self._log_metrics(log_fn, exclude=self.count)
+            t1 = time.perf_counter()
+            for name, v in meter.update(step_this_run, t1 - t0, tokens).items():
+                self.record_metric(name, v)
+            t0 = t1
+        torch.cuda.synchronize()
+        self._log_metrics(log_fn)
 
     # ------------------------------------------------------------------ checkpoint
     def save_checkpoint(self, path: str, data_loader=None, tokens_seen: Optional[int] = None) -> None:

@@ -331,3 +331,44 @@ def test_checkpoint_round_trip_resumes_the_run(tmp_path):
         small = TransformerRecipe.tiny_llama()
         small.num_layers = 2
         Trainer(small.build(batch_size=B, sequence_length=S), AdamWConfig(lr=sched)).load_checkpoint(path)
+
+
+def test_fit_loop_logs_every_step_once_with_losses_of_a_manual_run():
+    """Trainer.fit (training loop of src/olmax/train/trainer.py:531-637): every step is logged exactly
+    once and in order, one step late; the logged losses, learning rates and gradient norms are those
+    of the same run driven by hand; throughput follows TPS = BPS x tokens with the averages from the
+    10th step on."""
+    say("fit loop")
+    from olmax_amd import AdamWConfig, Trainer, TransformerRecipe, WarmupCosineDecaySchedule, data
+    hcfg = TransformerRecipe.tiny_llama()
+    B, S, steps = 2, 128, 12
+    ocfg = ref.ModelConfig(vocab=4096, d_model=256, n_layers=4, n_heads=4, n_kv_heads=4, head_dim=64, hidden=1024,
+                           eps=1e-6, rope_theta=1e4)
+    P = ref.init_params(ocfg, seed=5)
+    sched = WarmupCosineDecaySchedule(3, 9, 1e-3, 1e-5, 1e-5)
+    kw = dict(vocab_size=4096, sequence_length=S, global_batch_size_instances=2 * B, total_batches=steps + 3, num_microbatches=2)
+
+    def fresh():
+        m = hcfg.build(batch_size=B, sequence_length=S)
+        m.load_state_dict(P)
+        return Trainer(m, AdamWConfig(lr=sched, weight_decay=0.1, max_grad_norm=1.0), overlap_optimizer=False)
+
+    tr = fresh()
+    want = []
+    for i, batch in enumerate(data.DataLoader(3, **kw)):
+        if i == steps:
+            break
+        lr = tr.optim.lr_at(tr.count)
+        loss = tr.train_batch([(x.reshape(-1), y.reshape(-1)) for x, y in batch]).item()
+        want.append((loss, lr, tr.grad_norm))
+
+    tr2 = fresh()
+    logged = []
+    tr2.fit(data.DataLoader(3, **kw), max_steps=steps, log_fn=lambda s, m: logged.append((s, m)))
+    assert tr2.count == steps and [s for s, _ in logged] == list(range(1, steps + 1))
+    for (s, m), (loss, lr, gn) in zip(logged, want):
+        assert m["optim/lr"] == pytest.approx(lr, rel=1e-6)
+        assert m["train/loss"] == pytest.approx(loss, rel=1e-3 if s > 1 else 1e-6)
+        assert m["optim/g_norm"] == pytest.approx(gn, rel=2e-2)
+        assert m["throughput/TPS"] == pytest.approx(m["throughput/BPS"] * 2 * B * S)
+        assert ("throughput/TPS average" in m) == (s >= 10)
