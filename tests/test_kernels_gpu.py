@@ -82,6 +82,31 @@ def test_gemm_brute_force_tiny_and_strided():
     assert maxrel(got, av.double().cpu() @ bv.double().cpu().t()) < 6e-3
 
 
+@pytest.mark.parametrize("al,bl", [(0, 0), (0, 1), (1, 1), (1, 0)])
+@pytest.mark.parametrize("M,N,K", [(2048, 4096, 192), (2048, 4096, 256), (4096, 4352, 64)])
+def test_gemm_256_tiles_row_strided_operands(M, N, K, al, bl):
+    """The 256x256-tile kernel (>= 128 tiles) with every operand a column slice of a wider buffer
+    (leading dimensions that are not the row length, 16-byte aligned offsets), odd and even k-tile
+    counts, a strided residual and a strided output; the 272-tile case is cut into whole rounds
+    plus a remainder.  Against a float64 product of the same bf16 values."""
+    ops = _ops()
+    say(f"gemm 256-tile strided M{M} N{N} K{K} a{al} b{bl}")
+    ar, ac = (M, K) if al == 0 else (K, M)
+    br, bc = (N, K) if bl == 0 else (K, N)
+    big_a = bfr(ar, ac + 72, seed=11).cuda(); big_b = bfr(br, bc + 40, seed=12, scale=0.05).cuda()
+    av, bv = big_a[:, 8:8 + ac], big_b[:, 24:24 + bc]
+    big_r = bfr(M, N + 16, seed=13).cuda(); rv = big_r[:, 8:8 + N]
+    af = av.double() if al == 0 else av.double().t()
+    bf_ = bv.double() if bl == 0 else bv.double().t()
+    want = (af @ bf_.t()).cpu()
+    got = ops.gemm(av, bv, a_layout=al, b_layout=bl)
+    assert maxrel(got, want) < 6e-3
+    out = torch.zeros(M, N + 24, device="cuda", dtype=BF)
+    ops.gemm(av, bv, a_layout=al, b_layout=bl, residual=rv, out=out[:, 16:16 + N])
+    assert maxrel(out[:, 16:16 + N], want + rv.double().cpu()) < 6e-3
+    assert not out[:, :16].any() and not out[:, 16 + N:].any()  # nothing written outside the view
+
+
 def test_gemm_rejects_bad_arguments():
     ops = _ops()
     from olmax_amd._lib import OlmaxHipError
