@@ -28,6 +28,7 @@ GEMM_TRAFFIC_BYTES = {
     256 | 1 << 12 | 1 << 13: 1.566e9,               # A_KC,B_KC (qkv, LM head)
     256 | 1 << 12 | 1 << 13 | 1 << 14: 0.767e9,     # A_KC,B_KC + residual (o, down)
     256 | 1 << 12 | 1 << 13 | 1 << 16: 2.586e9,     # A_KC,B_KC + GLU epilogue (gate+up)
+    256 | 1 << 12 | 1 << 13 | 1 << 17: 1.566e9,     # A_KC,B_KC + RoPE epilogue (q|k|v; same operands as the plain kernel)
 }
 
 
@@ -140,7 +141,7 @@ def main():
         k = keys[i]
         name = "gemm_bf16_kernel<tile%d,%s,%s%s%s%s>" % (k & 0xfff, "A_KC" if k >> 12 & 1 else "A_MC", "B_KC" if k >> 13 & 1 else "B_NC",
                                                          ",res" if k >> 14 & 1 else "", ",f32out" if k >> 15 & 1 else "",
-                                                         ",glu" if k >> 16 & 1 else "")
+                                                         ",glu" if k >> 16 & 1 else ",rope" if k >> 17 & 1 else "")
         per.append({"kernel": name, "key": k, "launches": ln[i], "total_ms": ms[i], "avg_ms": ms[i] / ln[i],
                     "tflops": fl[i] / ms[i] / 1e9, "algorithmic_bytes_per_launch": by[i] / ln[i]})
     per.sort(key=lambda r: -r["total_ms"])

@@ -96,6 +96,17 @@ int32_t olmax_gemm_glu_bf16(olmax_stream_t stream, const void* X, const void* W,
                             int32_t M, int32_t F, int32_t K, int64_t ldx, int64_t ldw, int64_t ldgu,
                             int64_t ldact, int32_t act);
 
+/* ---- q|k|v projection with the rotary embedding fused into the GEMM epilogue:
+ * MultiheadSelfAttention.forward, src/olmax/nn/attention.py:270-274 (projections) and :298-300
+ * (RoPE on q and k, src/olmax/nn/rope.py:99-115), for recipes without QK-norm.
+ * out[M, N] = X W^T with W = [Wq; Wk; Wv] ([N, K], row stride ldw); the first rope_heads heads of
+ * 128 columns (q then k) leave rotated, position of row r = r % seq_len, cos/sin [seq_len, 64]
+ * fp32.  Equals olmax_gemm_bf16 followed by olmax_qk_rope_fwd in place (the path taken when the
+ * shape does not fit: M, N % 256, K % 64, rope_heads even, >= 128 tiles). */
+int32_t olmax_gemm_rope_bf16(olmax_stream_t stream, const void* X, const void* W, void* out, int32_t M, int32_t N,
+                             int32_t K, int64_t ldx, int64_t ldw, int64_t ldo, const float* cos_t,
+                             const float* sin_t, int32_t seq_len, int32_t rope_heads);
+
 /* ---- Gated MLP activation: GatedMLP.forward, src/olmax/nn/mlp.py:69-73:
  * out = act(gate) * up, act 0 = silu, 1 = tanh-approximated gelu (jax.nn.gelu default,
  * src/olmax/nn/transformer/layer.py:133). */

@@ -61,12 +61,21 @@ std::mutex g_prof_mu;
 // and 128 up rows, arranged in LDS so that every wave owns the gate AND the up columns of the
 // same 32 features; the epilogue writes act = f(gate) * up ([M, F], leading dimension ldr) and,
 // when Cv is given, gate|up ([M, 2F]) as the plain GEMM would.  N is F in that mode.
-template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32, int GLU = 0>
+//
+// EPI == 3 is the fused q|k|v projection + rotary embedding: columns below rope_cols are heads of
+// 128 that leave the kernel rotated (out = x cos + rotate_half(x) sin in fp32 on the bf16-rounded
+// projection, as the separate RoPE kernel computes it); a wave's 64 columns are one half of a
+// head and its neighbour (wave ^ 1) holds the other, so the rotation reads both from the LDS
+// staging of the epilogue.  The position of a row is row % seq_len; cos/sin are [seq_len, 64] fp32.
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32, int EPI = 0>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm_bf16_kernel(
     const bf16* __restrict__ A, const bf16* __restrict__ B, void* __restrict__ Cv,
     const bf16* __restrict__ R, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-    int64_t ldr, int tiles_m, int tiles_n, int c_vec) {
-  static_assert(GLU == 0 || (BN == 256 && WN == 64 && B_KC && !HAS_RES && !OUT_F32), "GLU epilogue: 256-wide NT tiles only");
+    int64_t ldr, int tiles_m, int tiles_n, int c_vec, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int seq_len, int rope_cols) {
+  constexpr int GLU = (EPI == 1 || EPI == 2) ? EPI : 0;
+  constexpr bool ROPE = EPI == 3;
+  static_assert(EPI == 0 || (BN == 256 && WN == 64 && B_KC && !HAS_RES && !OUT_F32), "fused epilogues: 256-wide NT tiles only");
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int TM = WM / 16, TN = WN / 16;  // accumulators of 16x16 per wave
   constexpr int WAVES_N = BN / WN;
@@ -434,6 +443,37 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
         *reinterpret_cast<u32x2*>(ws + row * 128 + ((chunk ^ kswz(row)) << 4) + ((g16e & 1) << 3)) = pk.u;
       }
     bf16* C = reinterpret_cast<bf16*>(Cv);
+    if (ROPE && n0 < rope_cols) {  // uniform over the block: rope_cols is a multiple of 256
+      // Rotation on the way out.  Every wave has staged its half-heads; now wave w takes rows
+      // 32w .. 32w+31 of the whole 256-column block, two rows (2 x 512 B) per instruction, so
+      // that the four lanes of a row that need the same cos/sin entry (two heads x two halves)
+      // sit in one instruction and share one request: the tables cost 128 KB per block, not 512.
+      __syncthreads();
+#pragma unroll 4
+      for (int t = 0; t < 16; t++) {
+        const int row = wave * 32 + t * 2 + (lane_e >> 5);      // row of the block
+        const int c32 = lane_e & 31, chunk = c32 & 7;            // 16-byte chunk of the 512-byte row
+        const int lrow = row & (WM - 1);                         // row inside the staging region
+        const unsigned char* own = smem + ((row / WM) * WAVES_N + (c32 >> 3)) * (WM * 128) + lrow * 128 + ((chunk ^ kswz(lrow)) << 4);
+        const unsigned char* oth = smem + ((row / WM) * WAVES_N + ((c32 >> 3) ^ 1)) * (WM * 128) + lrow * 128 + ((chunk ^ kswz(lrow)) << 4);
+        Pack8 xo, xp, o;
+        xo.u = *reinterpret_cast<const u32x4*>(own);
+        xp.u = *reinterpret_cast<const u32x4*>(oth);
+        const int pos = (m0 + row) % seq_len;
+        const float* cp = cos_t + (int64_t)pos * 64 + chunk * 8;
+        const float* sp = sin_t + (int64_t)pos * 64 + chunk * 8;
+        const f32x4 c0 = *reinterpret_cast<const f32x4*>(cp), c1 = *reinterpret_cast<const f32x4*>(cp + 4);
+        const f32x4 s0 = *reinterpret_cast<const f32x4*>(sp), s1 = *reinterpret_cast<const f32x4*>(sp + 4);
+        const float sign = (c32 & 8) ? 1.f : -1.f;  // first half: x1 cos - x2 sin; second: x2 cos + x1 sin
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const float cs = e < 4 ? c0[e & 3] : c1[e & 3], sn = e < 4 ? s0[e & 3] : s1[e & 3];
+          o.e[e] = f2bf(bf2f(xo.e[e]) * cs + sign * bf2f(xp.e[e]) * sn);
+        }
+        *reinterpret_cast<u32x4*>(C + (int64_t)(m0 + row) * ldc + n0 + c32 * 8) = o.u;
+      }
+      return;
+    }
 #pragma unroll
     for (int t = 0; t < WM / 8; t++) {
       const int row = t * 8 + (lane_e >> 3), chunk = lane_e & 7;
@@ -514,7 +554,7 @@ int launch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16
   // vector epilogue: 16-byte stores to C, 8-byte loads from R
   const int c_vec = aligned16(C) && ldc % 8 == 0 && (!R || ((((uintptr_t)R) & 7) == 0 && ldr % 4 == 0));
   hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(NT), SMEM, s, A, B, C, R, M, N, K, lda, ldb, ldc,
-                     ldr, tm, tn, c_vec);
+                     ldr, tm, tn, c_vec, (const float*)nullptr, (const float*)nullptr, 1, 0);
   if (g_prof_on) {
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 2.0 * M * N * K;
@@ -546,7 +586,7 @@ int launch_glu(hipStream_t s, const bf16* A, const bf16* B, bf16* gu, bf16* act,
   }
   const int c_vec = (((uintptr_t)act) & 7) == 0 && ldact % 4 == 0 && (!gu || ((((uintptr_t)gu) & 7) == 0 && ldgu % 4 == 0 && F % 4 == 0));
   hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(512), SMEM, s, A, B, (void*)gu, (const bf16*)act, M, F, K, lda, ldb,
-                     ldgu, ldact, tm, tn, c_vec);
+                     ldgu, ldact, tm, tn, c_vec, (const float*)nullptr, (const float*)nullptr, 1, 0);
   if (g_prof_on) {
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 4.0 * M * F * K;
@@ -583,7 +623,7 @@ extern "C" void olmax_gemm_profile_begin(void) {
 }
 // Stop recording, wait for the recorded events and aggregate per kernel instantiation.
 // keys/ms/flops/launches: host arrays of `cap` entries; returns the number of distinct keys.
-// key = tile | a_layout<<12 | b_layout<<13 | has_residual<<14 | out_f32<<15 | glu_epilogue<<16,
+// key = tile | a_layout<<12 | b_layout<<13 | has_residual<<14 | out_f32<<15 | glu_epilogue<<16 | rope_epilogue<<17,
 // with a_layout / b_layout bit SET when the operand is reduction-contiguous.  flops / bytes:
 // algorithmic totals (2MNK; every operand and the result moved once).
 extern "C" int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, double* bytes, int64_t* launches,
@@ -703,6 +743,58 @@ extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void
   if (!a_kc && !b_kc) GO(false, false);
   GO(false, true);
 #undef GO
+}
+
+extern "C" int32_t olmax_qk_rope_fwd(hipStream_t stream, const void* x, void* y, const void* w, const float* cos_t,
+                                     const float* sin_t, int64_t tokens, int32_t heads, int32_t head_dim, int32_t seq_len,
+                                     int64_t ldx, int64_t ldy, float eps);
+
+// q|k|v projection with the rotary embedding of the q and k heads in the GEMM epilogue:
+// out[M, N] = X W^T, then columns [0, rope_heads * 128) are rotated head by head (head_dim 128,
+// position of row r = r % seq_len, cos/sin [seq_len, 64] fp32).  Equals olmax_gemm_bf16 followed
+// by olmax_qk_rope_fwd in place on those columns, which is also what it falls back to when the
+// shape does not fit the fused kernel.
+extern "C" int32_t olmax_gemm_rope_bf16(hipStream_t stream, const void* X, const void* W, void* out, int32_t M, int32_t N,
+                                        int32_t K, int64_t ldx, int64_t ldw, int64_t ldo, const float* cos_t,
+                                        const float* sin_t, int32_t seq_len, int32_t rope_heads) {
+  OLMAX_CHECK(X && W && out && cos_t && sin_t, OLMAX_ERR_ARG, "olmax_gemm_rope_bf16: null operand");
+  OLMAX_CHECK(M > 0 && N > 0 && K > 0 && seq_len > 0 && rope_heads >= 0 && (int64_t)rope_heads * 128 <= N, OLMAX_ERR_SHAPE,
+              "olmax_gemm_rope_bf16: bad shape (M %d N %d K %d seq_len %d rope_heads %d)", M, N, K, seq_len, rope_heads);
+  OLMAX_CHECK(ldx >= K && ldw >= K && ldo >= N, OLMAX_ERR_SHAPE, "olmax_gemm_rope_bf16: leading dimension smaller than row length");
+  const bool fits = aligned16(X) && aligned16(W) && aligned16(out) && aligned16(cos_t) && aligned16(sin_t) && ldx % 8 == 0 &&
+                    ldw % 8 == 0 && ldo % 8 == 0 && K % BK == 0 && M % 256 == 0 && N % 256 == 0 && rope_heads % 2 == 0 &&
+                    (int64_t)(M / 256) * (N / 256) >= 128 && !g_force_tile;
+  if (fits) {
+    constexpr int SMEM = 2 * (256 + 256) * BK * 2;
+    auto kern = gemm_bf16_kernel<256, 256, 128, 64, true, true, false, false, 3>;
+    static bool attr_set = false;
+    if (!attr_set) {
+      (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+      attr_set = true;
+    }
+    const int tm = M / 256, tn = N / 256;
+    ProfRec rec{};
+    if (g_prof_on) {
+      (void)hipEventCreate(&rec.e0);
+      (void)hipEventCreate(&rec.e1);
+      (void)hipEventRecord(rec.e0, stream);
+    }
+    hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(512), SMEM, stream, (const bf16*)X, (const bf16*)W, out, (const bf16*)nullptr, M,
+                       N, K, ldx, ldw, ldo, (int64_t)0, tm, tn, 1, cos_t, sin_t, seq_len, rope_heads * 128);
+    if (g_prof_on) {
+      (void)hipEventRecord(rec.e1, stream);
+      rec.flops = 2.0 * M * N * K;
+      rec.bytes = 2.0 * ((double)M * K + (double)N * K + (double)M * N);
+      rec.key = 256 | (1 << 12) | (1 << 13) | (1 << 17);
+      std::lock_guard<std::mutex> lk(g_prof_mu);
+      g_prof.push_back(rec);
+    }
+    OLMAX_LAUNCH_CHECK();
+    return OLMAX_OK;
+  }
+  int rc = olmax_gemm_bf16(stream, X, W, out, nullptr, M, N, K, ldx, ldw, ldo, 0, 0, 0, 0);
+  if (rc || rope_heads == 0) return rc;
+  return olmax_qk_rope_fwd(stream, out, out, nullptr, cos_t, sin_t, M, rope_heads, 128, seq_len, ldo, ldo, 0.f);
 }
 
 extern "C" int32_t olmax_glu_fwd(hipStream_t stream, const void* gate, const void* up, void* out, int64_t T, int32_t F,

@@ -146,7 +146,12 @@ int block_forward(hipStream_t s, const olmax_model_config* c, const olmax_block_
     RC(olmax_rmsnorm_fwd(s, x, lt == 0 ? w->attn_norm : w->attn_in_norm, a.xn, m.T, m.d, m.d, m.d, eps));
     attn_in = a.xn;
   }
-  RC(lin_fwd(s, attn_in, m.d, w->wqkv, m.d, m.QKV, a.qkv, m.QKV, nullptr, 0, m.T));
+  // without QK-norm the rotary embedding rides in the projection's epilogue (head_dim 128)
+  const bool rope_in_gemm = !c->qk_norm && m.D == 128;
+  if (rope_in_gemm)
+    RC(olmax_gemm_rope_bf16(s, attn_in, w->wqkv, a.qkv, (int)m.T, m.QKV, m.d, m.d, m.d, m.QKV, cos_t, sin_t, m.S, m.H + m.K));
+  else
+    RC(lin_fwd(s, attn_in, m.d, w->wqkv, m.d, m.QKV, a.qkv, m.QKV, nullptr, 0, m.T));
   const bf16 *qp, *kp;
   int64_t ldqk;
   if (c->qk_norm) {
@@ -157,7 +162,7 @@ int block_forward(hipStream_t s, const olmax_model_config* c, const olmax_block_
     kp = a.qkr + m.HD;
   } else {
     ldqk = m.QKV;
-    RC(olmax_qk_rope_fwd(s, a.qkv, a.qkv, nullptr, cos_t, sin_t, m.T, m.H + m.K, m.D, m.S, m.QKV, m.QKV, eps));
+    if (!rope_in_gemm) RC(olmax_qk_rope_fwd(s, a.qkv, a.qkv, nullptr, cos_t, sin_t, m.T, m.H + m.K, m.D, m.S, m.QKV, m.QKV, eps));
     qp = a.qkv;
     kp = a.qkv + m.HD;
   }

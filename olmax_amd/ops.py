@@ -168,6 +168,21 @@ def gated_mlp_in(x, w_gate_up, act: str = "silu", gate_up_out=None, save_gate_up
     return out, gate_up_out
 
 
+def qkv_rope_proj(x, w_qkv, cos, sin, *, rope_heads: int, seq_len: int, out=None):
+    """q|k|v projection with RoPE applied to the first `rope_heads` heads (q then k, head_dim 128)
+    in the GEMM epilogue (reference src/olmax/nn/attention.py:270-274, 298-300).  Returns [T, N]."""
+    _need_gpu(x, w_qkv, cos, sin)
+    x = _rows2d(x)
+    T, d = x.shape
+    N = w_qkv.shape[0]
+    if out is None:
+        out = torch.empty(T, N, device=x.device, dtype=BF16)
+    check(_L().olmax_gemm_rope_bf16(stream_ptr(), ptr(x), ptr(w_qkv), ptr(out), i32(T), i32(N), i32(d), i64(x.stride(0)),
+                                    i64(w_qkv.stride(0)), i64(out.stride(0)), ptr(cos), ptr(sin), i32(seq_len),
+                                    i32(rope_heads)))
+    return out
+
+
 def glu_bwd(gate, up, dh, act: str = "silu", dgate=None, dup=None):
     _need_gpu(gate, up, dh)
     gate, up, dh = _rows2d(gate), _rows2d(up), _rows2d(dh)

@@ -222,6 +222,29 @@ def test_gated_mlp_in_fused_epilogue(act, T, F, d):
         assert maxrel(act_fused, want) < 2e-2
 
 
+@pytest.mark.parametrize("T,S,H,KH,d", [(4096, 1024, 8, 8, 256), (8192, 4096, 6, 2, 192), (512, 256, 2, 2, 128), (8192, 2048, 5, 3, 128)])
+def test_qkv_projection_with_rope_in_the_epilogue(T, S, H, KH, d):
+    """The q|k|v GEMM with RoPE in its epilogue must equal GEMM + qk_rope_fwd (in place on the q and
+    k heads) bit for bit: same projection tile, same fp32 rotation of the bf16-rounded values; v is
+    untouched.  Cases: fused shapes (>= 128 tiles, even head count), a small one and an odd head
+    count that take the unfused path, and the oracle on one of them."""
+    ops = _ops()
+    say(f"qkv+rope T{T} S{S} H{H} K{KH} d{d}")
+    N = (H + 2 * KH) * 128
+    x = bfr(T, d, seed=1).cuda(); w = bfr(N, d, seed=2, scale=d ** -0.5).cuda()
+    cos, sin = ops.rope_tables(S, 128, 10000.0, "cuda")
+    plain = ops.gemm(x, w)
+    want = plain.clone()
+    ops.qk_rope_fwd(want[:, :(H + KH) * 128], cos, sin, heads=H + KH, head_dim=128, seq_len=S, out=want[:, :(H + KH) * 128])
+    got = ops.qkv_rope_proj(x, w, cos, sin, rope_heads=H + KH, seq_len=S)
+    assert torch.equal(got[:, (H + KH) * 128:], plain[:, (H + KH) * 128:])
+    assert torch.equal(got, want)
+    if T <= 512:
+        q = ref.linear_fwd(x.cpu().double(), w.cpu().double(), rt)[:, :(H + KH) * 128].reshape(T // S, S, H + KH, 128)
+        rq = ref.rope_fwd(q, *ref.rope_tables(S, 128, 10000.0), rt)
+        assert maxrel(got[:, :(H + KH) * 128], rq.reshape(T, -1)) < 2e-2
+
+
 ATTN_CASES = [
     # B, S, H, KH, D, window, softcap
     (2, 256, 4, 4, 128, None, 0.0),
