@@ -67,6 +67,61 @@ def cpu_baseline(sample_tokens: int = 512):
     }
 
 
+def hbm_kernels(T: int, d: int, F: int, heads: int, V: int):
+    """Achieved HBM bandwidth of the memory-bound kernels of the step, each timed alone with HIP
+    events on the launch stream at the 7B shapes, against the 8 TB/s peak.  Bytes are algorithmic
+    (every operand and result moved once).  Each kernel cycles over enough distinct buffers that
+    nothing it reads is left in the 256 MB Infinity Cache from its previous launch."""
+    import torch
+
+    from olmax_amd import ops
+    BF = torch.bfloat16
+    dev = "cuda"
+    out = []
+
+    def timed(name, nbytes, footprint, make, call, iters=24):
+        nset = max(2, int(768e6 // footprint) + 1)
+        sets = [make() for _ in range(nset)]
+        for i in range(4):
+            call(sets[i % nset])
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(iters):
+            call(sets[i % nset])
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / iters
+        out.append({"kernel": name, "algorithmic_bytes": nbytes, "us": us, "achieved_GBps": nbytes / us / 1e3,
+                    "frac_of_8TBps": nbytes / us / 1e3 / 8000.0})
+        del sets
+        torch.cuda.empty_cache()
+
+    rnd = lambda *sh: torch.randn(*sh, device=dev).to(BF)
+    w = torch.ones(d, device=dev, dtype=BF)
+    timed("rmsnorm_fwd [T,d]", 4 * T * d, 4 * T * d, lambda: (rnd(T, d), torch.empty(T, d, device=dev, dtype=BF)),
+          lambda b: ops.rms_norm_fwd(b[0], w, 1e-6, out=b[1]))
+    dw = torch.zeros(d, device=dev)
+    timed("rmsnorm_bwd + residual grad [T,d]", 8 * T * d, 8 * T * d,
+          lambda: (rnd(T, d), rnd(T, d), rnd(T, d), torch.empty(T, d, device=dev, dtype=BF)),
+          lambda b: ops.rms_norm_bwd(b[0], w, b[1], 1e-6, dres=b[2], dw=dw, out=b[3]))
+    timed("glu_bwd (silu) [T,F]", 10 * T * F, 10 * T * F,
+          lambda: (rnd(T, 2 * F), rnd(T, F), torch.empty(T, 2 * F, device=dev, dtype=BF)),
+          lambda b: ops.glu_bwd(b[0][:, :F], b[0][:, F:], b[1], "silu", dgate=b[2][:, :F], dup=b[2][:, F:]))
+    cos, sin = ops.rope_tables(4096, 128, 5e5, dev)
+    timed("qk_rope_bwd in place [T,heads*128]", 4 * T * heads * 128, 2 * T * heads * 128, lambda: (rnd(T, heads * 128),),
+          lambda b: ops.qk_rope_bwd(b[0], cos, sin, heads=heads, head_dim=128, seq_len=4096, out=b[0]))
+    labels = torch.randint(0, V, (T,), device=dev, dtype=torch.int32)
+    timed("cross_entropy fwd+bwd in place [T,V] bf16", 4 * T * V, 2 * T * V, lambda: (rnd(T, V),),
+          lambda b: ops.cross_entropy(b[0], labels, inplace=True), iters=8)
+    n = 202_383_360  # parameters of one 7B block
+    timed("adamw (bf16 grads, bf16 copy out) one block", 28 * n, 30 * n,
+          lambda: (torch.zeros(n, device=dev), rnd(n), torch.zeros(n, device=dev), torch.zeros(n, device=dev),
+                   torch.empty(n, device=dev, dtype=BF)),
+          lambda b: ops.adamw_(b[0], b[1], b[2], b[3], step=1, lr=1e-4, shadow=b[4]), iters=8)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -74,6 +129,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-checkpoint", action="store_true", help="keep activations instead of full-block recompute")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-hbm-kernels", action="store_true", help="skip the stand-alone timing of the memory-bound kernels")
     ap.add_argument("--no-keep-activations-leg", action="store_true", help="skip the extra measurement without recompute")
     ap.add_argument("--no-overlap", action="store_true", help="run AdamW after the backward pass instead of overlapping it on a second stream")
     ap.add_argument("--profiler-ranges", action="store_true", help="emit roctx ranges per layer and phase (for rocprofv3 --marker-trace)")
@@ -190,6 +246,10 @@ def main():
         out["keep_activations"] = {"value": tps2, "unit": "tokens/s", "ms_per_step": dt2 / args.steps * 1e3,
                                    "mfu_bf16": tps2 * flops_tok / PEAK_BF16,
                                    "note": "activation_checkpointing off (reference recipe default); not the headline config"}
+    if not args.no_hbm_kernels:
+        del trainer, model
+        torch.cuda.empty_cache()
+        out["hbm_kernels"] = hbm_kernels(T, cfg.d_model, 11008, 64, cfg.vocab_size)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
