@@ -129,7 +129,10 @@ void olmax_range_pop(void);
 
 // GLU activations (GatedMLP, reference src/olmax/nn/mlp.py:69-73): jax.nn.silu and the tanh
 // form of jax.nn.gelu; shared by the elementwise GLU kernels and the GEMM's fused epilogue.
-__device__ __forceinline__ float act_silu(float g) { return g / (1.f + __expf(-g)); }
+// silu(g) = g * sigmoid(g); the reciprocal is the hardware approximation (1 ulp), not the ~10-instruction
+// IEEE division: the result is rounded to bf16 right away, and in the GEMM epilogue every
+// vector instruction is time the matrix pipe idles.
+__device__ __forceinline__ float act_silu(float g) { return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)); }
 constexpr float GELU_C = 0.7978845608028654f;  // sqrt(2/pi)
 __device__ __forceinline__ float act_gelu(float g) {
   return 0.5f * g * (1.f + tanhf(GELU_C * (g + 0.044715f * g * g * g)));
