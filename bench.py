@@ -99,6 +99,11 @@ def hbm_kernels(T: int, d: int, F: int, heads: int, V: int):
 
     rnd = lambda *sh: torch.randn(*sh, device=dev).to(BF)
     w = torch.ones(d, device=dev, dtype=BF)
+    # yardstick: what a plain device-to-device copy of the same size reaches under the same conditions
+    timed("copy [T,d] bf16 (torch copy_, for scale)", 4 * T * d, 4 * T * d, lambda: (rnd(T, d), torch.empty(T, d, device=dev, dtype=BF)),
+          lambda b: b[1].copy_(b[0]))
+    timed("copy [T,F] x 5 arrays of bf16 (torch copy_, for scale)", 4 * T * F * 5 // 2, 4 * T * F * 5 // 2,
+          lambda: (rnd(T, 5 * F // 2), torch.empty(T, 5 * F // 2, device=dev, dtype=BF)), lambda b: b[1].copy_(b[0]))
     timed("rmsnorm_fwd [T,d]", 4 * T * d, 4 * T * d, lambda: (rnd(T, d), torch.empty(T, d, device=dev, dtype=BF)),
           lambda b: ops.rms_norm_fwd(b[0], w, 1e-6, out=b[1]))
     dw = torch.zeros(d, device=dev)
