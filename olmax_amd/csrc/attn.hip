@@ -162,11 +162,6 @@ __device__ __forceinline__ bf16x8 pack_bf16x8(const f32x16& a, int base) {
   return r;
 }
 
-__device__ __forceinline__ float fast_tanh(float x) {
-  // tanh(x) = 1 - 2 / (exp(2x) + 1); exact enough in fp32 for |x| up to saturation
-  const float e = __expf(2.f * x);
-  return 1.f - 2.f / (e + 1.f);
-}
 
 // ---------------------------------------------------------------------------------------
 // Forward.  grid = ceil(S/128)*H*B workgroups (see decode_wg); 256 threads; wave w owns queries i0+32w .. +31.

@@ -18,7 +18,7 @@ __device__ __forceinline__ float act_silu_grad(float g) {
   return s * (1.f + g * (1.f - s));
 }
 __device__ __forceinline__ float act_gelu_grad(float g) {
-  const float t = tanhf(GELU_C * (g + 0.044715f * g * g * g));
+  const float t = fast_tanh(GELU_C * (g + 0.044715f * g * g * g));
   return 0.5f * (1.f + t) + 0.5f * g * (1.f - t * t) * GELU_C * (1.f + 3.f * 0.044715f * g * g);
 }
 

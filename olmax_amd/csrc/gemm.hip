@@ -379,6 +379,55 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   if (GLU) {
     bf16* act = const_cast<bf16*>(R);
     bf16* gu = reinterpret_cast<bf16*>(Cv);
+    if (c_vec == 2) {
+      // Whole-line stores through LDS.  A wave's 128 x 32 features are half a line per row, so the
+      // block's 256 x 128 output is staged wave by wave (64-byte rows, 16-byte chunks XOR-swizzled
+      // by (row >> 2) & 3) and written out by rows: wave w takes rows 32w .. 32w+31, four rows of
+      // 256 B per instruction.  First act, then (when kept for the backward pass) gate and up.
+      constexpr int REG = WM * 64;  // bytes of one wave's staging region
+      __syncthreads();              // every wave is done reading the operand stages
+#pragma unroll 1
+      for (int pass = 0; pass < (gu ? 2 : 1); pass++) {
+        if (pass) __syncthreads();  // the previous pass has been read back
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++) {
+            const int row = i * 16 + l16e;
+            unsigned char* dst = smem + wave * REG + row * 64 + ((((j << 1) | (g16e >> 1)) ^ ((row >> 2) & 3)) << 4) + ((g16e & 1) << 3);
+            Pack4 pa, pg, pu;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              // same roundings as the unfused path: gate and up are bf16 arrays, so is f(gate)
+              pg.e[r] = f2bf(acc[i][j][r]);
+              pu.e[r] = f2bf(acc[i][j + 2][r]);
+              const float gf = bf2f(pg.e[r]);
+              const float a = bf2f(f2bf(GLU == 2 ? act_gelu(gf) : act_silu(gf)));
+              pa.e[r] = f2bf(a * bf2f(pu.e[r]));
+            }
+            if (pass == 0) {
+              *reinterpret_cast<u32x2*>(dst) = pa.u;
+            } else {
+              *reinterpret_cast<u32x2*>(dst) = pg.u;
+              *reinterpret_cast<u32x2*>(dst + 8 * REG) = pu.u;
+            }
+          }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const int row = wave * 32 + t * 4 + (lane_e >> 4), c = lane_e & 15;
+          const int lrow = row & (WM - 1);
+          const unsigned char* src = smem + ((row / WM) * WAVES_N + (c >> 2)) * REG + lrow * 64 + (((c & 3) ^ ((lrow >> 2) & 3)) << 4);
+          if (pass == 0) {
+            *reinterpret_cast<u32x4*>(act + (int64_t)(m0 + row) * ldr + n0 + c * 8) = *reinterpret_cast<const u32x4*>(src);
+          } else {
+            *reinterpret_cast<u32x4*>(gu + (int64_t)(m0 + row) * ldc + n0 + c * 8) = *reinterpret_cast<const u32x4*>(src);
+            *reinterpret_cast<u32x4*>(gu + (int64_t)(m0 + row) * ldc + N + n0 + c * 8) = *reinterpret_cast<const u32x4*>(src + 8 * REG);
+          }
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -584,7 +633,9 @@ int launch_glu(hipStream_t s, const bf16* A, const bf16* B, bf16* gu, bf16* act,
     (void)hipEventCreate(&rec.e1);
     (void)hipEventRecord(rec.e0, s);
   }
-  const int c_vec = (((uintptr_t)act) & 7) == 0 && ldact % 4 == 0 && (!gu || ((((uintptr_t)gu) & 7) == 0 && ldgu % 4 == 0 && F % 4 == 0));
+  // 2: 16-byte stores of whole lines through LDS; 1: 8-byte stores straight from the accumulators
+  const int c_vec = (aligned16(act) && ldact % 8 == 0 && (!gu || (aligned16(gu) && ldgu % 8 == 0 && F % 8 == 0))) ? 2
+                    : ((((uintptr_t)act) & 7) == 0 && ldact % 4 == 0 && (!gu || ((((uintptr_t)gu) & 7) == 0 && ldgu % 4 == 0 && F % 4 == 0)));
   hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(512), SMEM, s, A, B, (void*)gu, (const bf16*)act, M, F, K, lda, ldb,
                      ldgu, ldact, tm, tn, c_vec, (const float*)nullptr, (const float*)nullptr, 1, 0);
   if (g_prof_on) {
