@@ -78,6 +78,11 @@ int32_t olmax_rmsnorm_bwd(olmax_stream_t stream, const void* x, const void* w, c
  * x/y: [tokens, heads*head_dim] views (in place allowed); position = token % seq_len;
  * cos/sin: fp32 [seq_len, head_dim/2] (precompute_freqs_cis, rope.py:118-145).
  * w != NULL: y = rope(bf16(rms_norm_per_head(x, w))). */
+/* cos/sin tables [seq_len, head_dim/2] fp32: precompute_freqs_cis, src/olmax/nn/rope.py:118-145
+ * (freqs = 1 / theta^(2i/D), t = arange(seq_len), their outer product and cos/sin all in fp32,
+ * rope.py:127-133; RotaryPositionalEmbedding.get_freqs_cis / warmup_cache, rope.py:82-97). */
+int32_t olmax_rope_tables(olmax_stream_t stream, float* cos_t, float* sin_t, int32_t seq_len,
+                          int32_t head_dim, float theta);
 int32_t olmax_qk_rope_fwd(olmax_stream_t stream, const void* x, void* y, const void* w,
                           const float* cos_t, const float* sin_t, int64_t tokens, int32_t heads,
                           int32_t head_dim, int32_t seq_len, int64_t ldx, int64_t ldy, float eps);

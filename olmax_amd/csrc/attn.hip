@@ -809,12 +809,14 @@ extern "C" int32_t olmax_attn_fwd(hipStream_t stream, const void* q, const void*
   return OLMAX_OK;
 }
 
-// Workspace: delta [B,H,S] fp32; the generic (head_dim != 128) path additionally needs two
-// fp32 [B*S, KH*D] accumulators.
+// Workspace: delta [B,H,S] fp32, then two fp32 [B*S, KH*D] accumulators for the generic path.
+// Which path runs depends on head_dim AND on the alignment of the operands (a head_dim-128 call
+// on unaligned views takes the generic path), which this query cannot see: it always returns the
+// size that covers both.
+static int64_t attn_delta_bytes(int32_t B, int32_t S, int32_t H) { return ((int64_t)B * H * S * 4 + 255) / 256 * 256; }
+static int64_t attn_acc_bytes(int32_t B, int32_t S, int32_t KH, int32_t D) { return ((int64_t)B * S * KH * D * 4 + 255) / 256 * 256; }
 extern "C" int64_t olmax_attn_bwd_workspace_bytes(int32_t B, int32_t S, int32_t H, int32_t KH, int32_t D) {
-  int64_t n = ((int64_t)B * H * S * 4 + 255) / 256 * 256;
-  if (D != 128) n += 2 * (((int64_t)B * S * KH * D * 4 + 255) / 256 * 256);
-  return n;
+  return attn_delta_bytes(B, S, H) + 2 * attn_acc_bytes(B, S, KH, D);
 }
 
 extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void* k, const void* v,
@@ -825,7 +827,7 @@ extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void*
                                   int64_t lddv, int32_t window, float softcap) {
   OLMAX_CHECK(q && k && v && o && lse && d_o && dq && dk && dv && workspace, OLMAX_ERR_ARG, "olmax_attn_bwd: null pointer");
   OLMAX_CHECK(B > 0 && S > 0 && H > 0 && KH > 0 && D > 0 && H % KH == 0, OLMAX_ERR_SHAPE, "olmax_attn_bwd: bad shape");
-  OLMAX_CHECK(workspace_bytes >= olmax_attn_bwd_workspace_bytes(B, S, H, KH, D) && (((uintptr_t)workspace) & 255) == 0, OLMAX_ERR_WORKSPACE, "olmax_attn_bwd: workspace too small or not 256-byte aligned");
+  OLMAX_CHECK(workspace_bytes >= attn_delta_bytes(B, S, H) && (((uintptr_t)workspace) & 255) == 0, OLMAX_ERR_WORKSPACE, "olmax_attn_bwd: workspace too small or not 256-byte aligned");
   OLMAX_CHECK(ldq >= (int64_t)H * D && ldo >= (int64_t)H * D && lddo >= (int64_t)H * D && lddq >= (int64_t)H * D && ldk >= (int64_t)KH * D && ldv >= (int64_t)KH * D && lddk >= (int64_t)KH * D && lddv >= (int64_t)KH * D, OLMAX_ERR_SHAPE, "olmax_attn_bwd: row stride smaller than heads*head_dim");
   const float scale = 1.f / sqrtf((float)D);
   const bf16 *qp = (const bf16*)q, *kp = (const bf16*)k, *vp = (const bf16*)v, *op = (const bf16*)o, *gop = (const bf16*)d_o;
@@ -854,8 +856,11 @@ extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void*
     }
   } else {
     OLMAX_CHECK(D <= 256 && (size_t)S * 8 <= 65536, OLMAX_ERR_SHAPE, "olmax_attn_bwd: generic path supports head_dim <= 256 and seq_len <= 8192");
-    const int64_t accb = ((int64_t)B * S * KH * D * 4 + 255) / 256 * 256;
-    float* dkf = (float*)((char*)workspace + ((int64_t)B * H * S * 4 + 255) / 256 * 256);
+    const int64_t accb = attn_acc_bytes(B, S, KH, D);
+    OLMAX_CHECK(workspace_bytes >= attn_delta_bytes(B, S, H) + 2 * accb, OLMAX_ERR_WORKSPACE,
+                "olmax_attn_bwd: the generic path (head_dim != 128, or operands not 16-byte aligned) needs %ld workspace bytes",
+                (long)(attn_delta_bytes(B, S, H) + 2 * accb));
+    float* dkf = (float*)((char*)workspace + attn_delta_bytes(B, S, H));
     float* dvf = (float*)((char*)dkf + accb);
     { int rc = olmax_fill_zero(stream, dkf, 2 * accb); if (rc) return rc; }
     hipLaunchKernelGGL(attn_bwd_generic, dim3(S, H, B), dim3(64), (size_t)S * 8, stream, qp, kp, vp, op, gop, lse, (bf16*)dq, dkf, dvf, S, H, KH, D, ldq, ldk, ldv, ldo, lddo, lddq, scale, window, softcap);

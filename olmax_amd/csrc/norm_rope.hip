@@ -426,6 +426,21 @@ __global__ __launch_bounds__(64) void qk_rope_bwd_generic(
   }
 }
 
+// cos/sin of position * theta^(-2i/D), every intermediate in fp32 and in the reference's order
+// of operations (precompute_freqs_cis, src/olmax/nn/rope.py:127-133): exponent = (2i)/D,
+// freq = 1 / theta^exponent, angle = float(position) * freq.
+__global__ __launch_bounds__(256) void rope_tables_kernel(float* __restrict__ cos_t, float* __restrict__ sin_t,
+                                                          int seq_len, int half, float head_dim, float theta) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)seq_len * half) return;
+  const int p = (int)(idx / half), i = (int)(idx % half);
+  const float exponent = (float)(2 * i) / head_dim;
+  const float freq = 1.0f / powf(theta, exponent);
+  const float ang = (float)p * freq;
+  cos_t[idx] = cosf(ang);
+  sin_t[idx] = sinf(ang);
+}
+
 int grid_for(int64_t work_items, int per_block, int cap) {
   int64_t g = (work_items + per_block - 1) / per_block;
   if (g > cap) g = cap;
@@ -547,6 +562,20 @@ extern "C" int32_t olmax_qk_rope_bwd(hipStream_t stream, const void* dy, void* d
     OLMAX_CHECK(head_dim <= 512, OLMAX_ERR_SHAPE, "olmax_qk_rope_bwd: head_dim > 512 unsupported");
     hipLaunchKernelGGL(qk_rope_bwd_generic, dim3((unsigned)(tokens * heads)), dim3(64), 0, stream, dyp, dxp, (const bf16*)x, (const bf16*)w, dw, cos_t, sin_t, tokens, heads, head_dim, seq_len, lddy, lddx, ldx, eps);
   }
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
+
+// cos/sin tables [seq_len, head_dim/2] fp32 for the rotary embedding, formed in fp32 as the
+// reference forms them.
+extern "C" int32_t olmax_rope_tables(hipStream_t stream, float* cos_t, float* sin_t, int32_t seq_len,
+                                     int32_t head_dim, float theta) {
+  OLMAX_CHECK(cos_t && sin_t, OLMAX_ERR_ARG, "olmax_rope_tables: null pointer");
+  OLMAX_CHECK(seq_len > 0 && head_dim > 0 && head_dim % 2 == 0 && theta > 0.f, OLMAX_ERR_SHAPE, "olmax_rope_tables: bad shape or theta");
+  const int half = head_dim / 2;
+  const int64_t n = (int64_t)seq_len * half;
+  hipLaunchKernelGGL(rope_tables_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, cos_t, sin_t, seq_len, half,
+                     (float)head_dim, theta);
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
 }

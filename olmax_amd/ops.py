@@ -101,11 +101,15 @@ def rms_norm_bwd(x, w, dy, eps: float, dres=None, dw: Optional[torch.Tensor] = N
 
 # ----------------------------------------------------------------------------- RoPE (+ head-wise QK-norm)
 def rope_tables(seq_len: int, head_dim: int, theta: float, device) -> Tuple[torch.Tensor, torch.Tensor]:
-    """cos/sin [S, D/2] fp32 (olmax.nn.rope.precompute_freqs_cis): fp32 angles, as the reference."""
-    inv = 1.0 / (theta ** (torch.arange(0.0, head_dim, 2, dtype=torch.float64) / head_dim))
-    ang = torch.outer(torch.arange(seq_len, dtype=torch.float64), inv).to(torch.float32).to(torch.float64)
-    return (torch.cos(ang).to(torch.float32).to(device).contiguous(),
-            torch.sin(ang).to(torch.float32).to(device).contiguous())
+    """cos/sin [S, D/2] fp32 on the GPU (olmax.nn.rope.precompute_freqs_cis, rope.py:118-145),
+    computed by the library in fp32 throughout, as the reference does."""
+    device = torch.device(device)
+    if device.type != "cuda":
+        raise _lib.OlmaxHipError("olmax_amd ops run on the GPU only; there is no CPU fallback")
+    cos = torch.empty(seq_len, head_dim // 2, device=device, dtype=torch.float32)
+    sin = torch.empty_like(cos)
+    check(_L().olmax_rope_tables(stream_ptr(), ptr(cos), ptr(sin), i32(seq_len), i32(head_dim), f32(theta)))
+    return cos, sin
 
 
 def qk_rope_fwd(x, cos, sin, *, heads: int, head_dim: int, seq_len: int, w=None, eps: float = 1e-6, out=None):

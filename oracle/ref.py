@@ -69,12 +69,17 @@ def rms_norm_bwd(x: Tensor, w: Optional[Tensor], dy: Tensor, eps: float, rt=_id)
 
 # --------------------------------------------------------------------------- RoPE
 def rope_tables(seq_len: int, head_dim: int, theta: float, dtype=torch.float32):
-    """src/olmax/nn/rope.py:118-145 — cos/sin of outer(arange(S), theta^(-2i/D)), [S, D/2]."""
-    inv = 1.0 / (theta ** (torch.arange(0.0, head_dim, 2, dtype=torch.float64) / head_dim))
-    ang = torch.outer(torch.arange(seq_len, dtype=torch.float64), inv)
-    # the reference forms the angles in fp32; cos/sin are stored in fp32
-    ang = ang.to(torch.float32).to(torch.float64) if dtype == torch.float32 else ang
-    return torch.cos(ang).to(dtype), torch.sin(ang).to(dtype)
+    """src/olmax/nn/rope.py:118-145 — cos/sin of outer(arange(S), theta^(-2i/D)), [S, D/2].
+
+    The reference forms `freqs`, `t` and their outer product in its default float type
+    (fp32: `jnp.arange(0.0, head_dim, 2)`, `jnp.arange(float(end))`, rope.py:127-130) and only
+    the cos/sin results take `dtype`; every intermediate below is therefore an array of
+    `dtype` itself (fp32 by default; fp64 gives the exact closed form for checks)."""
+    exponent = torch.arange(0.0, head_dim, 2, dtype=dtype) / head_dim
+    freqs = 1.0 / torch.pow(torch.tensor(theta, dtype=dtype), exponent)
+    t = torch.arange(float(seq_len), dtype=dtype)
+    ang = torch.outer(t, freqs)
+    return torch.cos(ang), torch.sin(ang)
 
 
 def rope_fwd(x: Tensor, cos: Tensor, sin: Tensor, rt=_id) -> Tensor:
@@ -348,7 +353,8 @@ class ModelConfig:
     hidden: int
     layer_type: str = "pre"        # "pre" | "reordered" | "gemma"
     act: str = "silu"              # "silu" | "gelu"
-    qk_norm: bool = False          # head-wise QK-norm
+    qk_norm: bool = False          # QK-norm on (src/olmax/nn/attention.py:239-253)
+    qk_norm_headwise: bool = True  # True: weight [D] per head (:293-296); False: full width (:281-284)
     eps: float = 1e-6
     rope_theta: float = 10000.0
     rope_theta_layers: Optional[list] = None   # per-layer override
@@ -382,8 +388,10 @@ def init_params(cfg: ModelConfig, seed: int = 0, std: float = 0.02, dtype=torch.
         p[pre + "attention.v_proj.weight"] = n(K * D, d)
         p[pre + "attention.o_proj.weight"] = n(d, H * D)
         if cfg.qk_norm:
-            p[pre + "attention.q_norm.weight"] = torch.ones(D, dtype=dtype)
-            p[pre + "attention.k_norm.weight"] = torch.ones(D, dtype=dtype)
+            # full width: the reference sizes both weights n_heads*head_dim (attention.py:239-253),
+            # which only fits k when n_kv_heads == n_heads; k's own width is used here
+            p[pre + "attention.q_norm.weight"] = torch.ones(D if cfg.qk_norm_headwise else H * D, dtype=dtype)
+            p[pre + "attention.k_norm.weight"] = torch.ones(D if cfg.qk_norm_headwise else K * D, dtype=dtype)
         p[pre + "mlp.gate_proj.weight"] = n(F, d)
         p[pre + "mlp.up_proj.weight"] = n(F, d)
         p[pre + "mlp.down_proj.weight"] = n(d, F)
@@ -408,13 +416,16 @@ class _Tape:
 def _attn_fwd(cfg, P, pre, l, x, tape, rt):
     B, S, d = x.shape
     H, K, D = cfg.n_heads, cfg.n_kv_heads, cfg.head_dim
-    q = linear_fwd(x, P[pre + "attention.q_proj.weight"], rt).reshape(B, S, H, D)
-    k = linear_fwd(x, P[pre + "attention.k_proj.weight"], rt).reshape(B, S, K, D)
+    q = linear_fwd(x, P[pre + "attention.q_proj.weight"], rt)
+    k = linear_fwd(x, P[pre + "attention.k_proj.weight"], rt)
     v = linear_fwd(x, P[pre + "attention.v_proj.weight"], rt).reshape(B, S, K, D)
+    if cfg.qk_norm and cfg.qk_norm_headwise:  # after the reshape (src/olmax/nn/attention.py:293-296)
+        q, k = q.reshape(B, S, H, D), k.reshape(B, S, K, D)
     tape["q0"], tape["k0"] = q, k
-    if cfg.qk_norm:  # head-wise (src/olmax/nn/attention.py:293-296)
+    if cfg.qk_norm:  # full width: before the reshape (src/olmax/nn/attention.py:281-284)
         q = rms_norm_fwd(q, P[pre + "attention.q_norm.weight"], cfg.eps, rt)
         k = rms_norm_fwd(k, P[pre + "attention.k_norm.weight"], cfg.eps, rt)
+    q, k = q.reshape(B, S, H, D), k.reshape(B, S, K, D)
     cos, sin = rope_tables(S, D, cfg.theta(l))
     q = rope_fwd(q, cos, sin, rt)
     k = rope_fwd(k, cos, sin, rt)
@@ -435,8 +446,8 @@ def _attn_bwd(cfg, P, pre, l, dy, tape, G, rt):
     dq = rope_bwd(dq, tape["cos"], tape["sin"], rt)
     dk = rope_bwd(dk, tape["cos"], tape["sin"], rt)
     if cfg.qk_norm:
-        dq, G[pre + "attention.q_norm.weight"] = rms_norm_bwd(tape["q0"], P[pre + "attention.q_norm.weight"], dq, cfg.eps, rt)
-        dk, G[pre + "attention.k_norm.weight"] = rms_norm_bwd(tape["k0"], P[pre + "attention.k_norm.weight"], dk, cfg.eps, rt)
+        dq, G[pre + "attention.q_norm.weight"] = rms_norm_bwd(tape["q0"], P[pre + "attention.q_norm.weight"], dq.reshape(tape["q0"].shape), cfg.eps, rt)
+        dk, G[pre + "attention.k_norm.weight"] = rms_norm_bwd(tape["k0"], P[pre + "attention.k_norm.weight"], dk.reshape(tape["k0"].shape), cfg.eps, rt)
     x = tape["attn_in"]
     dxq, G[pre + "attention.q_proj.weight"] = linear_bwd(x, P[pre + "attention.q_proj.weight"], dq.reshape(B, S, H * D), rt)
     dxk, G[pre + "attention.k_proj.weight"] = linear_bwd(x, P[pre + "attention.k_proj.weight"], dk.reshape(B, S, K * D), rt)
@@ -545,22 +556,55 @@ def model_loss_and_grads(cfg: ModelConfig, P: dict, ids: Tensor, labels: Tensor,
     return loss, G
 
 
+def decay_mask(names, no_decay) -> dict:
+    """OptimConfig.build_weight_decay_mask (src/olmax/optim/config.py:94-122): a leaf decays
+    unless its dotted path matches one of the fnmatch patterns."""
+    return {n: not any(_fnmatch(n, pat) for pat in (no_decay or ())) for n in names}
+
+
+def clip_by_global_norm(G: dict, max_norm: float):
+    """clip_grads_by_global_norm (src/olmax/optim/utils.py:22-38; norm from get_global_norm,
+    src/olmax/jax_utils.py:88-102): g <- (g / max(max_norm, ||g||)) * max_norm over ALL leaves
+    together.  Returns (clipped, norm)."""
+    norm = torch.sqrt(sum((g.double() ** 2).sum() for g in G.values()))
+    clamped = max(float(max_norm), float(norm))
+    return {n: (g / clamped) * max_norm for n, g in G.items()}, norm
+
+
+def multisteps_mean(grads: list) -> dict:
+    """optax.MultiSteps' accumulator (third party; built at src/olmax/optim/config.py:153-154):
+    the k micro-batch gradients enter a running mean acc += (g - acc) / (j + 1)."""
+    acc = None
+    for j, G in enumerate(grads):
+        acc = dict(G) if acc is None else {n: acc[n] + (G[n] - acc[n]) / (j + 1) for n in acc}
+    return acc
+
+
+def apply_adamw(master: dict, opt: dict, G: dict, *, step: int, lr: float, b1=0.9, b2=0.999, eps=1e-8,
+                wd=1e-4, no_decay=("embedding.weight",)) -> None:
+    """step_optimizer (src/olmax/train/trainer.py:742-757): optax.adamw with the weight-decay
+    mask of AdamWConfig.build (src/olmax/optim/config.py:136-148) on every leaf, in place."""
+    mask = decay_mask(master, no_decay)
+    for name in master:
+        master[name], opt["m"][name], opt["v"][name] = adamw_step(
+            master[name], G[name].to(master[name].dtype), opt["m"][name], opt["v"][name],
+            step=step, lr=lr, b1=b1, b2=b2, eps=eps, wd=wd if mask[name] else 0.0)
+
+
+def _compute_params(master: dict, compute_bf16: bool):
+    if compute_bf16:
+        return {k: bf16_round(v) for k, v in master.items()}, bf16_round
+    return master, _id
+
+
 def train_step(cfg: ModelConfig, master: dict, opt: dict, ids, labels, *, step: int, lr: float,
                b1=0.9, b2=0.999, eps=1e-8, wd=1e-4, no_decay=("embedding.weight",),
                compute_bf16: bool = False):
     """process_microbatch (src/olmax/train/trainer.py:723-777): cast master → compute dtype,
     loss+grads, grads → fp32, AdamW on the fp32 master copy.  `opt` = {"m":…, "v":…}."""
-    if compute_bf16:
-        P = {k: bf16_round(v) for k, v in master.items()}
-        rt = bf16_round
-    else:
-        P, rt = master, _id
+    P, rt = _compute_params(master, compute_bf16)
     loss, G = model_loss_and_grads(cfg, P, ids, labels, rt)
-    for name in master:
-        decay = 0.0 if any(_fnmatch(name, pat) for pat in no_decay) else wd
-        master[name], opt["m"][name], opt["v"][name] = adamw_step(
-            master[name], G[name].to(master[name].dtype), opt["m"][name], opt["v"][name],
-            step=step, lr=lr, b1=b1, b2=b2, eps=eps, wd=decay)
+    apply_adamw(master, opt, G, step=step, lr=lr, b1=b1, b2=b2, eps=eps, wd=wd, no_decay=no_decay)
     return loss, G
 
 
@@ -569,30 +613,19 @@ def train_batch(cfg: ModelConfig, master: dict, opt: dict, batch, *, step: int, 
                 compute_bf16: bool = False, max_grad_norm=None):
     """train_batch (src/olmax/train/trainer.py:779-807) with the optimizer wrapped in
     optax.MultiSteps(k) (src/olmax/optim/config.py:153-154; third party, restated from its
-    documentation: parity unpinned): gradients are cast to fp32 (trainer.py:738), the k
-    micro-batches enter the running mean acc += (g - acc) / (j + 1), the clip
-    (src/olmax/optim/utils.py:22-38) and AdamW act once, on the mean, and the reported loss is the
-    mean of the micro-batch losses.  `batch` = [(ids, labels), ...]."""
-    if compute_bf16:
-        P = {k: bf16_round(v) for k, v in master.items()}
-        rt = bf16_round
-    else:
-        P, rt = master, _id
-    acc, losses = None, []
-    for j, (ids, labels) in enumerate(batch):
+    documentation): gradients are cast to fp32 (trainer.py:738), the k micro-batches enter the
+    running mean, the clip (src/olmax/optim/utils.py:22-38) and AdamW act once, on the mean, and
+    the reported loss is the mean of the micro-batch losses.  `batch` = [(ids, labels), ...]."""
+    P, rt = _compute_params(master, compute_bf16)
+    grads, losses = [], []
+    for ids, labels in batch:
         loss, G = model_loss_and_grads(cfg, P, ids, labels, rt)
         losses.append(loss)
-        G = {n: g.to(torch.float32).to(master[n].dtype) for n, g in G.items()}
-        acc = G if acc is None else {n: acc[n] + (G[n] - acc[n]) / (j + 1) for n in acc}
+        grads.append({n: g.to(torch.float32).to(master[n].dtype) for n, g in G.items()})
+    acc = multisteps_mean(grads)
     if max_grad_norm is not None:
-        norm = torch.sqrt(sum((g.double() ** 2).sum() for g in acc.values()))
-        scale = max_grad_norm / max(max_grad_norm, float(norm))
-        acc = {n: g * scale for n, g in acc.items()}
-    for name in master:
-        decay = 0.0 if any(_fnmatch(name, pat) for pat in no_decay) else wd
-        master[name], opt["m"][name], opt["v"][name] = adamw_step(
-            master[name], acc[name], opt["m"][name], opt["v"][name],
-            step=step, lr=lr, b1=b1, b2=b2, eps=eps, wd=decay)
+        acc, _ = clip_by_global_norm(acc, max_grad_norm)
+    apply_adamw(master, opt, acc, step=step, lr=lr, b1=b1, b2=b2, eps=eps, wd=wd, no_decay=no_decay)
     return sum(losses) / len(losses), acc
 
 

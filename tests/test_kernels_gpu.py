@@ -146,6 +146,30 @@ def test_rmsnorm_empty_and_strided():
     assert maxrel(y, ref.rms_norm_fwd(v.double().cpu(), None, 1e-5)) < 1e-2
 
 
+@pytest.mark.parametrize("S,D,theta", [(4096, 128, 500000.0), (4096, 128, 10000.0), (4096, 128, 1e6), (512, 64, 10000.0), (77, 16, 3.5)])
+def test_rope_tables_follow_the_reference_arithmetic(S, D, theta):
+    """olmax_rope_tables against (a) the exact closed form cos/sin(p * theta^(-2i/D)) in float64 and
+    (b) the oracle's fp32 table (torch-CPU arithmetic in the reference's order of operations,
+    src/olmax/nn/rope.py:127-133).  Both comparisons are by tolerance: the kernel and the oracle are
+    two independent fp32 implementations (different powf / cosf), and an fp32 angle is only good
+    to a few ulp: |d angle| <= 4 * 2^-23 * angle (pow, reciprocal, product)."""
+    ops = _ops()
+    say(f"rope tables S{S} D{D} theta{theta}")
+    cos, sin = ops.rope_tables(S, D, theta, "cuda")
+    assert cos.shape == (S, D // 2) and cos.dtype == torch.float32
+    cos, sin = cos.cpu().double(), sin.cpu().double()
+    p = torch.arange(S, dtype=torch.float64)[:, None]
+    i = torch.arange(D // 2, dtype=torch.float64)[None, :]
+    ang = p * theta ** (-2.0 * i / D)
+    tol = 4 * 2.0 ** -23 * ang + 2.0 ** -22
+    assert ((cos - torch.cos(ang)).abs() <= tol).all() and ((sin - torch.sin(ang)).abs() <= tol).all()
+    rc, rs = ref.rope_tables(S, D, theta)
+    assert ((cos - rc.double()).abs() <= 2 * tol).all() and ((sin - rs.double()).abs() <= 2 * tol).all()
+    # positions are exact integers: frequency 0 (inv_freq == 1) must see the angle p itself
+    assert ((cos[:, 0] - torch.cos(p[:, 0])).abs() <= 2.0 ** -22).all()
+    assert torch.equal(cos[0], torch.ones(D // 2, dtype=torch.float64)) and torch.equal(sin[0], torch.zeros(D // 2, dtype=torch.float64))
+
+
 @pytest.mark.parametrize("D,heads,norm", [(128, 4, False), (128, 3, True), (64, 4, False), (16, 2, True)])
 def test_qk_rope(D, heads, norm):
     ops = _ops()
@@ -154,8 +178,7 @@ def test_qk_rope(D, heads, norm):
     x = bfr(B * S, heads * D, seed=1); dy = bfr(B * S, heads * D, seed=2)
     w = (1 + 0.1 * torch.randn(D, generator=torch.Generator().manual_seed(3))).to(BF) if norm else None
     cos, sin = ops.rope_tables(S, D, 500000.0, "cuda")
-    rc, rs = ref.rope_tables(S, D, 500000.0)
-    assert torch.equal(cos.cpu(), rc) and torch.equal(sin.cpu(), rs)  # positions/tables bit-exact
+    rc, rs = cos.cpu(), sin.cpu()  # the same table feeds kernel and oracle: this test is about the rotation
     y = ops.qk_rope_fwd(x.cuda(), cos, sin, heads=heads, head_dim=D, seq_len=S, w=None if w is None else w.cuda())
     x4 = x.double().reshape(B, S, heads, D)
     xn = rt(ref.rms_norm_fwd(x4, w.double(), 1e-6)) if norm else x4
@@ -179,7 +202,7 @@ def test_qk_rope_inplace_on_strided_qkv():
     cos, sin = ops.rope_tables(S, D, 1e4, "cuda")
     qv = qkv[:, : H * D]
     ops.qk_rope_fwd(qv, cos, sin, heads=H, head_dim=D, seq_len=S, out=qv)
-    rc, rs = ref.rope_tables(S, D, 1e4)
+    rc, rs = cos.cpu(), sin.cpu()
     want = ref.rope_fwd(orig[:, : H * D].double().cpu().reshape(B, S, H, D), rc.double(), rs.double()).reshape(B * S, H * D)
     assert maxrel(qkv[:, : H * D], want) < 1e-2
     assert torch.equal(qkv[:, H * D:], orig[:, H * D:])  # k, v untouched
@@ -241,7 +264,7 @@ def test_qkv_projection_with_rope_in_the_epilogue(T, S, H, KH, d):
     assert torch.equal(got, want)
     if T <= 512:
         q = ref.linear_fwd(x.cpu().double(), w.cpu().double(), rt)[:, :(H + KH) * 128].reshape(T // S, S, H + KH, 128)
-        rq = ref.rope_fwd(q, *ref.rope_tables(S, 128, 10000.0), rt)
+        rq = ref.rope_fwd(q, cos.cpu(), sin.cpu(), rt)
         assert maxrel(got[:, :(H + KH) * 128], rq.reshape(T, -1)) < 2e-2
 
 
@@ -258,7 +281,19 @@ ATTN_CASES = [
 ]
 
 
-@pytest.mark.parametrize("B,S,H,KH,D,window,softcap", ATTN_CASES)
+# The lengths the benchmark configurations run at: 64 key tiles per query tile, so the far-tile
+# skipping (window start, per-wave visibility), the lazy rescale over many tiles and the 1024-token
+# window of the local layers all bind.  The brute-force float64 oracle needs a few seconds each.
+ATTN_LONG_CASES = [
+    (1, 4096, 2, 1, 128, 1024, 0.0),
+    (1, 4096, 2, 1, 128, None, 50.0),
+    (1, 4096, 2, 2, 128, None, 0.0),
+    (1, 4000, 2, 1, 128, 1024, 0.0),    # ragged: last tiles partly outside the sequence
+    (1, 4096, 2, 1, 128, 4096, 50.0),   # window as long as the sequence: equals global causal
+]
+
+
+@pytest.mark.parametrize("B,S,H,KH,D,window,softcap", ATTN_CASES + ATTN_LONG_CASES)
 def test_attention_fwd_bwd(B, S, H, KH, D, window, softcap):
     ops = _ops()
     say(f"attn B{B} S{S} H{H} KH{KH} D{D} w{window} cap{softcap}")
@@ -288,6 +323,47 @@ def test_attention_on_strided_qkv_views():
     o, lse = ops.attn_fwd(q, k, v, B=B, S=S, H=H, KH=KH, D=D)
     o2, lse2 = ops.attn_fwd(q.contiguous(), k.contiguous(), v.contiguous(), B=B, S=S, H=H, KH=KH, D=D)
     assert torch.equal(o, o2) and torch.equal(lse, lse2)
+
+
+def test_attention_bwd_on_unaligned_views_stays_inside_its_workspace():
+    """head_dim 128 on views that are not 16-byte aligned takes the generic kernels, whose fp32
+    dK/dV accumulators live in the workspace behind delta: the size query must cover them, the
+    results must match the aligned call, and a workspace that only holds delta is refused on
+    the host (no launch)."""
+    import ctypes
+    ops = _ops()
+    from olmax_amd import _lib
+    from olmax_amd._lib import OlmaxHipError, i32, i64, f32, ptr, stream_ptr
+    say("attn bwd on unaligned D=128 views")
+    B, S, H, KH, D = 1, 64, 2, 1, 128
+    wide = lambda cols, seed: bfr(B * S, cols + 8, seed=seed).cuda()
+    bq, bk, bv, bdo = wide(H * D, 1), wide(KH * D, 2), wide(KH * D, 3), wide(H * D, 4)
+    q, k, v, do = bq[:, 4:4 + H * D], bk[:, 4:4 + KH * D], bv[:, 4:4 + KH * D], bdo[:, 4:4 + H * D]
+    assert q.data_ptr() % 16 == 8
+    o, lse = ops.attn_fwd(q, k, v, B=B, S=S, H=H, KH=KH, D=D)
+    qa, ka, va, doa = q.contiguous(), k.contiguous(), v.contiguous(), do.contiguous()
+    oa, lsea = ops.attn_fwd(qa, ka, va, B=B, S=S, H=H, KH=KH, D=D)
+    assert maxrel(o, oa) < 1e-2 and (lse - lsea).abs().max().item() < 2e-3
+    guard = torch.full((1 << 20,), 7, dtype=torch.uint8, device="cuda")  # allocated right behind the call's buffers
+    dq, dk, dv = ops.attn_bwd(q, k, v, o, lse, do, B=B, S=S, H=H, KH=KH, D=D)
+    dqa, dka, dva = ops.attn_bwd(qa, ka, va, oa, lsea, doa, B=B, S=S, H=H, KH=KH, D=D)
+    check_close(dq, dqa, "dq", tol=2e-2, cos=0.999); check_close(dk, dka, "dk", tol=2e-2, cos=0.999)
+    check_close(dv, dva, "dv", tol=2e-2, cos=0.999)
+    assert bool((guard == 7).all())
+    L = _lib.load()
+    L.olmax_attn_bwd_workspace_bytes.restype = ctypes.c_int64
+    full = L.olmax_attn_bwd_workspace_bytes(i32(B), i32(S), i32(H), i32(KH), i32(D))
+    delta_only = (B * H * S * 4 + 255) // 256 * 256
+    assert full >= delta_only + 2 * B * S * KH * D * 4
+    ws = torch.empty(delta_only, dtype=torch.uint8, device="cuda")
+    def call(qq, kk, vv, oo, dd, nbytes):
+        return L.olmax_attn_bwd(stream_ptr(), ptr(qq), ptr(kk), ptr(vv), ptr(oo), ptr(lse), ptr(dd), ptr(dq), ptr(dk), ptr(dv),
+                                ptr(ws), i64(nbytes), i32(B), i32(S), i32(H), i32(KH), i32(D), i64(qq.stride(0)), i64(kk.stride(0)),
+                                i64(vv.stride(0)), i64(oo.stride(0)), i64(dd.stride(0)), i64(dq.stride(0)), i64(dk.stride(0)),
+                                i64(dv.stride(0)), i32(-1), f32(0.0))
+    assert call(q, k, v, o, do, delta_only) == -5 and b"generic path" in L.olmax_last_error_string()
+    assert call(qa, ka, va, oa, doa, delta_only) == 0  # aligned operands: the MFMA path needs delta only
+    torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize("T,V,f32", [(33, 4096, False), (17, 1000, True), (8, 50, False), (5, 100352, False)])

@@ -254,7 +254,7 @@ def _autograd_model_loss(cfg, P, ids, labels):
 def test_model_grads_match_autograd(kind):
     cfg = ref.ModelConfig(vocab=37, d_model=16, n_layers=2, n_heads=4, n_kv_heads=2 if kind == "gemma" else 4,
                           head_dim=4, hidden=24, layer_type=kind, act="gelu" if kind == "gemma" else "silu",
-                          qk_norm=kind != "pre", windows=[3, None] if kind == "gemma" else None,
+                          qk_norm=kind != "pre", qk_norm_headwise=kind != "reordered", windows=[3, None] if kind == "gemma" else None,
                           rope_theta_layers=[1e4, 1e6] if kind == "gemma" else None,
                           attn_softcap=5.0 if kind == "gemma" else 0.0, final_softcap=3.0 if kind == "gemma" else 0.0,
                           tied=kind == "gemma")
@@ -271,10 +271,286 @@ def test_model_grads_match_autograd(kind):
         assert torch.allclose(G[n], g, atol=1e-10, rtol=1e-8), n
 
 
-def test_train_step_decreases_loss_and_masks_decay():
+def test_train_step_decreases_loss():
     cfg = ref.ModelConfig(vocab=50, d_model=16, n_layers=1, n_heads=2, n_kv_heads=2, head_dim=8, hidden=32)
     master = ref.init_params(cfg, seed=0)
     opt = {"m": {k: torch.zeros_like(v) for k, v in master.items()}, "v": {k: torch.zeros_like(v) for k, v in master.items()}}
     ids = torch.randint(0, 50, (2, 8)); labels = torch.randint(0, 50, (2, 8))
     losses = [ref.train_step(cfg, master, opt, ids, labels, step=s, lr=1e-2, wd=0.1)[0].item() for s in range(1, 6)]
     assert losses[-1] < losses[0]
+
+
+# ------------------------------------------------------------------------------------------
+# Pins for the pieces that used to be checked only against themselves: fp32 RoPE tables, the
+# three residual orderings, the weight-decay mask, global-norm clipping, the micro-batch
+# running mean and train_batch as a whole.  Each expected value below is built WITHOUT the
+# oracle function under test: closed forms, hand arithmetic, or torch's own textbook routines
+# (F.rms_norm, F.linear, F.scaled_dot_product_attention, torch.optim.AdamW, autograd).
+# ------------------------------------------------------------------------------------------
+def test_rope_tables_fp32_follow_reference_arithmetic():
+    """src/olmax/nn/rope.py:127-133 forms freqs, t and the outer product in fp32.  Against the
+    exact closed form cos(p * theta^(-2i/D)) the fp32 table may be off by the rounding of the
+    angle: |d angle| <= 4 ulp(fp32) of the angle (pow, reciprocal, product), i.e.
+    4 * 2^-23 * angle, plus the fp32 rounding of cos/sin itself."""
+    S, Dh, theta = 4096, 128, 500000.0
+    cos, sin = ref.rope_tables(S, Dh, theta)
+    assert cos.dtype == torch.float32 and cos.shape == (S, Dh // 2)
+    p = torch.arange(S, dtype=D64)[:, None]
+    i = torch.arange(Dh // 2, dtype=D64)[None, :]
+    ang = p * theta ** (-2.0 * i / Dh)
+    tol = 4 * 2.0 ** -23 * ang + 2.0 ** -23
+    assert ((cos.double() - torch.cos(ang)).abs() <= tol).all()
+    assert ((sin.double() - torch.sin(ang)).abs() <= tol).all()
+    # the tolerance is tight enough to tell fp32 angles from a dropped or doubled exponent:
+    wrong = p * theta ** (-1.0 * i / Dh)
+    assert ((cos.double() - torch.cos(wrong)).abs() > tol).any()
+    # frequency 0 has inv_freq == 1 exactly, so its angle is the integer position itself
+    assert torch.equal(cos[:, 0], torch.cos(torch.arange(S, dtype=torch.float32)))
+    assert torch.equal(cos[0], torch.ones(Dh // 2)) and torch.equal(sin[0], torch.zeros(Dh // 2))
+    # and the fp32 table is NOT the fp64 table rounded (the reference's angles carry fp32 error)
+    c64, _ = ref.rope_tables(S, Dh, theta, dtype=D64)
+    assert (cos.double() - c64).abs().max() > 1e-5
+
+
+def _torch_block(kind, P, pre, x, *, H, K, Dh, eps, theta, act, qk):
+    """One transformer block written from the reference's three forward() bodies
+    (src/olmax/nn/transformer/layer.py:86,90 / 108,112 / 175-177,181) and
+    MultiheadSelfAttention.forward (src/olmax/nn/attention.py:270-317) with torch's own
+    routines only; RoPE as a complex rotation of the (j, j + D/2) pairs."""
+    B, S, _ = x.shape
+
+    def norm(t, name):
+        return F.rms_norm(t, (t.shape[-1],), P[pre + name], eps)
+
+    def rope(t):
+        pos = torch.arange(S, dtype=D64)[:, None]
+        inv = theta ** (-torch.arange(0, Dh, 2, dtype=D64) / Dh)[None, :]
+        z = torch.polar(torch.ones(S, Dh // 2, dtype=D64), pos * inv)
+        tc = torch.complex(t[..., : Dh // 2], t[..., Dh // 2:]) * z[None, :, None, :]
+        return torch.cat([tc.real, tc.imag], -1)
+
+    def attn(t):
+        q = F.linear(t, P[pre + "attention.q_proj.weight"])
+        k = F.linear(t, P[pre + "attention.k_proj.weight"])
+        v = F.linear(t, P[pre + "attention.v_proj.weight"]).reshape(B, S, K, Dh)
+        if qk == "full":
+            q, k = norm(q, "attention.q_norm.weight"), norm(k, "attention.k_norm.weight")
+        q, k = q.reshape(B, S, H, Dh), k.reshape(B, S, K, Dh)
+        if qk == "head":
+            q, k = norm(q, "attention.q_norm.weight"), norm(k, "attention.k_norm.weight")
+        q, k = rope(q), rope(k)
+        o = F.scaled_dot_product_attention(q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3),
+                                           is_causal=True, enable_gqa=True).permute(0, 2, 1, 3)
+        return F.linear(o.reshape(B, S, H * Dh), P[pre + "attention.o_proj.weight"])
+
+    def mlp(t):
+        g = F.linear(t, P[pre + "mlp.gate_proj.weight"])
+        a = F.silu(g) if act == "silu" else F.gelu(g, approximate="tanh")
+        return F.linear(a * F.linear(t, P[pre + "mlp.up_proj.weight"]), P[pre + "mlp.down_proj.weight"])
+
+    if kind == "pre":
+        h = x + attn(norm(x, "attention_norm.weight"))
+        return h + mlp(norm(h, "mlp_norm.weight"))
+    if kind == "reordered":
+        h = x + norm(attn(x), "attention_norm.weight")
+        return h + norm(mlp(h), "mlp_norm.weight")
+    h = x + norm(attn(norm(x, "attention_input_norm.weight")), "attention_norm.weight")
+    return h + norm(mlp(norm(h, "mlp_input_norm.weight")), "mlp_norm.weight")
+
+
+def _random_block_params(cfg, seed):
+    g = torch.Generator().manual_seed(seed)
+    P = {}
+    for k, v in ref.init_params(cfg, seed=seed).items():
+        v = v.double()
+        P[k] = (1.0 + 0.3 * torch.randn(v.shape, generator=g, dtype=D64)) if "norm" in k else v * 10
+    return P
+
+
+@pytest.mark.parametrize("kind,qk", [("pre", "none"), ("pre", "full"), ("reordered", "head"), ("reordered", "none"),
+                                     ("gemma", "head"), ("gemma", "full")])
+def test_block_orderings_against_independent_torch_block(kind, qk):
+    H, K = (4, 4) if qk == "full" or kind == "pre" else (4, 2)
+    cfg = ref.ModelConfig(vocab=11, d_model=24, n_layers=2, n_heads=H, n_kv_heads=K, head_dim=6, hidden=40,
+                          layer_type=kind, act="gelu" if kind == "gemma" else "silu", qk_norm=qk != "none",
+                          qk_norm_headwise=qk != "full", eps=1e-5, rope_theta=777.0)
+    P = _random_block_params(cfg, seed=3)
+    x = torch.randn(2, 13, 24, dtype=D64)
+    for l in range(2):
+        want = _torch_block(kind, P, f"layers.{l}.", x, H=H, K=K, Dh=6, eps=1e-5, theta=777.0, act=cfg.act, qk=qk)
+        got, _ = ref.block_fwd(cfg, P, l, x)
+        # the oracle's block takes its cos/sin from the fp32 tables (as the reference does): 6e-8 relative
+        assert torch.allclose(got, want, atol=2e-6), (kind, qk, (got - want).abs().max())
+    # the three orderings are genuinely different functions of the same weights
+    if qk == "none" and kind != "gemma":
+        other = _torch_block("reordered" if kind == "pre" else "pre", P, "layers.0.", x, H=H, K=K, Dh=6, eps=1e-5,
+                             theta=777.0, act=cfg.act, qk=qk)
+        assert (ref.block_fwd(cfg, P, 0, x)[0] - other).abs().max() > 1e-3
+
+
+def test_block_ordering_scale_invariants():
+    """With eps = 0 a post-norm makes the block blind to the scale of o_proj / down_proj
+    (layer.py:108,112,175,181: the norm sits AFTER the sub-layer); in the pre-norm block
+    (layer.py:86,90) the sub-layer output is added as is, so its contribution scales."""
+    x = torch.randn(1, 9, 16, dtype=D64)
+    outs = {}
+    for kind in ("pre", "reordered", "gemma"):
+        cfg = ref.ModelConfig(vocab=5, d_model=16, n_layers=1, n_heads=2, n_kv_heads=2, head_dim=8, hidden=24,
+                              layer_type=kind, eps=0.0)
+        P = _random_block_params(cfg, seed=5)
+        y1, t1 = ref.block_fwd(cfg, P, 0, x)
+        P2 = dict(P)
+        P2["layers.0.attention.o_proj.weight"] = 3.0 * P["layers.0.attention.o_proj.weight"]
+        y2, t2 = ref.block_fwd(cfg, P2, 0, x)
+        outs[kind] = (y1, y2, t1["h"], t2["h"])
+    for kind in ("reordered", "gemma"):
+        y1, y2, _, _ = outs[kind]
+        assert torch.allclose(y1, y2, atol=1e-10), kind
+    _, _, h1, h2 = outs["pre"]
+    assert torch.allclose(h2 - x, 3.0 * (h1 - x), atol=1e-10)  # h = x + attn(...): linear in o_proj
+
+
+def test_decay_mask_patterns_and_pure_decay():
+    # the reference's own mask test (src/test/optim/config_test.py:36-47), names written out
+    names = [f"{m}.{p}" for m in ("gate_proj", "up_proj", "down_proj") for p in ("weight", "bias")]
+    mask = ref.decay_mask(names, ["gate_proj.bias", "down_proj.bias", "up_proj.bias"])
+    assert all(mask[f"{m}.weight"] is True and mask[f"{m}.bias"] is False for m in ("gate_proj", "up_proj", "down_proj"))
+    cfg = ref.ModelConfig(vocab=7, d_model=8, n_layers=2, n_heads=2, n_kv_heads=1, head_dim=4, hidden=12,
+                          layer_type="gemma", qk_norm=True)
+    master = {k: torch.full_like(v, 2.0).double() for k, v in ref.init_params(cfg).items()}
+    mask = ref.decay_mask(master, ["embedding.weight", "*norm.weight"])
+    assert mask["embedding.weight"] is False and mask["norm.weight"] is False
+    assert mask["layers.1.attention.q_norm.weight"] is False and mask["layers.0.mlp_input_norm.weight"] is False
+    assert mask["layers.0.mlp.up_proj.weight"] is True and mask["lm_head.proj.weight"] is True
+    assert sum(not v for v in mask.values()) == 2 + 2 * 6
+    # zero gradient: a masked leaf does not move, an unmasked one is p (1 - lr wd) exactly
+    opt = {"m": {k: torch.zeros_like(v) for k, v in master.items()}, "v": {k: torch.zeros_like(v) for k, v in master.items()}}
+    G = {k: torch.zeros_like(v) for k, v in master.items()}
+    ref.apply_adamw(master, opt, G, step=1, lr=0.1, wd=0.25, no_decay=["embedding.weight", "*norm.weight"])
+    for n, p in master.items():
+        want = 2.0 if not mask[n] else 2.0 * (1 - 0.1 * 0.25)
+        assert torch.equal(p, torch.full_like(p, want)), n
+
+
+def test_clip_by_global_norm_hand_examples():
+    """src/olmax/optim/utils.py:22-38: g * max_norm / max(max_norm, ||g||), one norm over all leaves."""
+    G = {"a": torch.tensor([3.0, 0.0], dtype=D64), "b": torch.tensor([[4.0]], dtype=D64)}  # ||g|| = 5
+    out, norm = ref.clip_by_global_norm(G, 1.0)
+    assert abs(float(norm) - 5.0) < 1e-15
+    assert torch.allclose(out["a"], torch.tensor([0.6, 0.0], dtype=D64), atol=1e-15) and abs(out["b"].item() - 0.8) < 1e-15
+    out, norm = ref.clip_by_global_norm(G, 10.0)  # below the threshold: factor 10 / max(10, 5) = 1
+    assert torch.allclose(out["a"], G["a"], atol=1e-15) and torch.allclose(out["b"], G["b"], atol=1e-15) and abs(float(norm) - 5.0) < 1e-15
+    out, _ = ref.clip_by_global_norm(G, 5.0)      # exactly at the threshold
+    assert torch.allclose(out["a"], G["a"], atol=1e-15)
+
+
+def test_multisteps_running_mean_is_the_plain_mean():
+    gs = [{"w": torch.tensor([1.0, -2.0], dtype=D64)}, {"w": torch.tensor([4.0, 0.0], dtype=D64)},
+          {"w": torch.tensor([-2.0, 8.0], dtype=D64)}, {"w": torch.tensor([5.0, 2.0], dtype=D64)}]
+    acc = ref.multisteps_mean(gs)
+    assert torch.allclose(acc["w"], torch.tensor([2.0, 2.0], dtype=D64), atol=1e-15)  # (1+4-2+5)/4, (-2+0+8+2)/4
+    assert torch.equal(ref.multisteps_mean(gs[:1])["w"], gs[0]["w"])
+
+
+def _tiny_train_setup(dtype):
+    cfg = ref.ModelConfig(vocab=23, d_model=16, n_layers=2, n_heads=2, n_kv_heads=1, head_dim=8, hidden=24,
+                          layer_type="gemma", act="gelu", qk_norm=True, tied=False)
+    g = torch.Generator().manual_seed(11)
+    master = {}
+    for k, v in ref.init_params(cfg, seed=2).items():
+        master[k] = ((1.0 + 0.2 * torch.randn(v.shape, generator=g)) if "norm" in k else v * 8).to(dtype)
+    batch = []
+    for j in range(3):
+        ids = torch.randint(0, 23, (2, 7), generator=g)
+        labels = torch.randint(0, 23, (2, 7), generator=g)
+        labels[0, : 2 * j] = -100  # different numbers of counted tokens per micro-batch
+        batch.append((ids, labels))
+    return cfg, master, batch
+
+
+def _zeros_like_opt(master):
+    return {"m": {k: torch.zeros_like(v) for k, v in master.items()}, "v": {k: torch.zeros_like(v) for k, v in master.items()}}
+
+
+def test_train_batch_of_identical_microbatches_equals_train_step():
+    cfg, master, batch = _tiny_train_setup(torch.float32)
+    m1 = {k: v.clone() for k, v in master.items()}
+    m2 = {k: v.clone() for k, v in master.items()}
+    o1, o2 = _zeros_like_opt(m1), _zeros_like_opt(m2)
+    ids, labels = batch[1]
+    l1, _ = ref.train_step(cfg, m1, o1, ids, labels, step=1, lr=1e-2, wd=0.1)
+    l2, _ = ref.train_batch(cfg, m2, o2, [(ids, labels)] * 3, step=1, lr=1e-2, wd=0.1)
+    assert torch.equal(l1, l2)
+    for n in m1:
+        assert torch.equal(m1[n], m2[n]) and torch.equal(o1["v"][n], o2["v"][n]), n
+
+
+@pytest.mark.parametrize("max_norm", [None, 0.05, 1e6])
+def test_train_batch_against_autograd_and_torch_adamw(max_norm):
+    """trainer.py:779-807 + optax.MultiSteps + the clip + masked AdamW, against a composition
+    that shares nothing with it: by linearity the mean of the micro-batch gradients is the
+    gradient of the mean of the micro-batch losses (autograd), the clip factor is computed by
+    hand, and torch.optim.AdamW (two param groups: decayed / not decayed) takes the step."""
+    cfg, master, batch = _tiny_train_setup(D64)
+    no_decay = ["embedding.weight", "*norm.weight"]
+    # --- independent composition
+    P = {k: v.clone().requires_grad_(True) for k, v in master.items()}
+    losses = [_autograd_model_loss(cfg, P, ids, labels) for ids, labels in batch]
+    mean_loss = sum(losses) / 3
+    names = list(P)
+    grads = dict(zip(names, torch.autograd.grad(mean_loss, [P[n] for n in names])))
+    norm = math.sqrt(sum(float((g ** 2).sum()) for g in grads.values()))
+    factor = 1.0 if max_norm is None else max_norm / max(max_norm, norm)
+    if max_norm == 0.05:
+        assert norm > 0.05  # the clip really binds in this case
+    import fnmatch
+    nd = [n for n in names if any(fnmatch.fnmatch(n, p) for p in no_decay)]
+    opt = torch.optim.AdamW([{"params": [P[n] for n in names if n not in nd], "weight_decay": 0.1},
+                             {"params": [P[n] for n in nd], "weight_decay": 0.0}], lr=1e-2, betas=(0.9, 0.95), eps=1e-3)
+    for n in names:
+        P[n].grad = grads[n] * factor
+    opt.step()
+    # --- the oracle
+    m2 = {k: v.clone() for k, v in master.items()}
+    o2 = _zeros_like_opt(m2)
+    loss, acc = ref.train_batch(cfg, m2, o2, batch, step=1, lr=1e-2, b1=0.9, b2=0.95, eps=1e-3, wd=0.1, no_decay=no_decay,
+                                max_grad_norm=max_norm)
+    assert abs(float(loss) - float(mean_loss.detach())) < 1e-7
+    for n in names:
+        # the oracle rounds gradients to fp32 (trainer.py:738) and rotates with fp32 cos/sin tables:
+        # ~1e-7 of the largest gradient; eps = 1e-3 keeps the Adam step Lipschitz (lr / eps = 10) in g
+        assert torch.allclose(acc[n], grads[n] * factor, rtol=1e-6, atol=1e-7), n
+        assert torch.allclose(m2[n], P[n].detach(), atol=2e-6), (n, (m2[n] - P[n].detach()).abs().max())
+    # and a second step, so that the moments carried in `opt` are exercised too
+    losses = [_autograd_model_loss(cfg, P, ids, labels) for ids, labels in batch]
+    grads = dict(zip(names, torch.autograd.grad(sum(losses) / 3, [P[n] for n in names])))
+    norm = math.sqrt(sum(float((g ** 2).sum()) for g in grads.values()))
+    factor = 1.0 if max_norm is None else max_norm / max(max_norm, norm)
+    for n in names:
+        P[n].grad = grads[n] * factor
+    opt.step()
+    ref.train_batch(cfg, m2, o2, batch, step=2, lr=1e-2, b1=0.9, b2=0.95, eps=1e-3, wd=0.1, no_decay=no_decay, max_grad_norm=max_norm)
+    for n in names:
+        assert torch.allclose(m2[n], P[n].detach(), atol=4e-6), (n, (m2[n] - P[n].detach()).abs().max())
+
+
+def test_train_step_against_autograd_and_torch_adamw():
+    """process_microbatch (trainer.py:723-777) in fp32 master / fp32 compute: same independent
+    composition with one micro-batch and the benchmark's mask (embedding.weight only)."""
+    cfg, master, batch = _tiny_train_setup(D64)
+    ids, labels = batch[2]
+    P = {k: v.clone().requires_grad_(True) for k, v in master.items()}
+    names = list(P)
+    opt = torch.optim.AdamW([{"params": [P[n] for n in names if n != "embedding.weight"], "weight_decay": 0.1},
+                             {"params": [P["embedding.weight"]], "weight_decay": 0.0}], lr=3e-3, betas=(0.9, 0.999), eps=1e-8)
+    m2 = {k: v.clone() for k, v in master.items()}
+    o2 = _zeros_like_opt(m2)
+    for step in (1, 2, 3):
+        loss = _autograd_model_loss(cfg, P, ids, labels)
+        for n, g in zip(names, torch.autograd.grad(loss, [P[n] for n in names])):
+            P[n].grad = g
+        opt.step()
+        l2, _ = ref.train_step(cfg, m2, o2, ids, labels, step=step, lr=3e-3, wd=0.1)
+        assert abs(float(l2) - float(loss.detach())) < 1e-7
+    for n in names:
+        assert torch.allclose(m2[n], P[n].detach(), atol=1e-5), n  # sign-like steps of 3e-3: any wrong term is >= 1e-3
