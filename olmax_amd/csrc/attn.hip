@@ -18,6 +18,7 @@
 // Backward is split in two deterministic kernels (no atomics): dK/dV with the key tile
 // stationary, dQ with the query tile stationary; each recomputes P from the saved LSE.
 #include "common.h"
+#include <mutex>
 #include <type_traits>
 
 extern "C" int32_t olmax_fill_zero(hipStream_t stream, void* p, int64_t nbytes);
@@ -776,6 +777,40 @@ bool fast_ok(int D, const void* q, const void* k, const void* v, const void* o, 
          ldk % 8 == 0 && ldv % 8 == 0 && ldo % 8 == 0;
 }
 
+bool bwd_fast_ok(const void* q, const void* k, const void* v, const void* o, const void* d_o, const void* dq, const void* dk,
+                 const void* dv, int D, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo, int64_t lddq,
+                 int64_t lddk, int64_t lddv) {
+  return fast_ok(D, q, k, v, o, ldq, ldk, ldv, ldo) && aligned16(d_o) && aligned16(dq) && aligned16(dk) && aligned16(dv) &&
+         lddo % 8 == 0 && lddq % 8 == 0 && lddk % 8 == 0 && lddv % 8 == 0;
+}
+
+// The three MFMA kernels of the backward pass (head_dim 128); delta: fp32 [B, H, S] scratch, fully
+// written by the first kernel before the other two read it.
+void launch_bwd_fast(hipStream_t stream, const bf16* qp, const bf16* kp, const bf16* vp, const bf16* op, const float* lse,
+                     const bf16* gop, bf16* dq, bf16* dk, bf16* dv, float* delta, int B, int S, int H, int KH, int64_t ldq,
+                     int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo, int64_t lddq, int64_t lddk, int64_t lddv, int window,
+                     float softcap) {
+  const float scale = 1.f / sqrtf(128.f);
+  const int64_t units = (int64_t)B * S * H;
+  hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((units + 15) / 16)), dim3(256), 0, stream, op, gop, delta, B, S, H, ldo, lddo);
+  dim3 gkv((unsigned)(((S + 127) / 128) * KH * B)), gq((unsigned)(((S + 127) / 128) * H * B));
+  constexpr int SM_KV = 2 * (2 * 32 * 256 + 256) + 128 * 256;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
+    (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
+    (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+  });
+  if (softcap > 0.f) {
+    hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, gkv, dim3(256), SM_KV, stream, qp, kp, vp, gop, lse, delta, dk, dv, S, H, KH, ldq, ldk, ldv, lddo, lddk, lddv, scale, window, softcap);
+    hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, gq, dim3(256), 65536, stream, qp, kp, vp, gop, lse, delta, dq, S, H, KH, ldq, ldk, ldv, lddo, lddq, scale, window, softcap);
+  } else {
+    hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, gkv, dim3(256), SM_KV, stream, qp, kp, vp, gop, lse, delta, dk, dv, S, H, KH, ldq, ldk, ldv, lddo, lddk, lddv, scale, window, softcap);
+    hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, gq, dim3(256), 65536, stream, qp, kp, vp, gop, lse, delta, dq, S, H, KH, ldq, ldk, ldv, lddo, lddq, scale, window, softcap);
+  }
+}
+
 }  // namespace
 
 // q [B*S, ldq] (head h at columns h*D..), k/v [B*S, ldk/ldv] (KH heads), o [B*S, ldo],
@@ -792,13 +827,14 @@ extern "C" int32_t olmax_attn_fwd(hipStream_t stream, const void* q, const void*
   const bf16 *qp = (const bf16*)q, *kp = (const bf16*)k, *vp = (const bf16*)v;
   if (fast_ok(D, q, k, v, o, ldq, ldk, ldv, ldo)) {
     dim3 grid((unsigned)(((S + 127) / 128) * H * B));
+    static std::once_flag once;
+    std::call_once(once, [] {
+      (void)hipFuncSetAttribute((const void*)attn_fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+      (void)hipFuncSetAttribute((const void*)attn_fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    });
     if (softcap > 0.f) {
-      static bool set = false;
-      if (!set) { (void)hipFuncSetAttribute((const void*)attn_fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536); set = true; }
       hipLaunchKernelGGL(attn_fwd_kernel<true>, grid, dim3(256), 65536, stream, qp, kp, vp, (bf16*)o, lse, S, H, KH, ldq, ldk, ldv, ldo, scale, window, softcap);
     } else {
-      static bool set = false;
-      if (!set) { (void)hipFuncSetAttribute((const void*)attn_fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536); set = true; }
       hipLaunchKernelGGL(attn_fwd_kernel<false>, grid, dim3(256), 65536, stream, qp, kp, vp, (bf16*)o, lse, S, H, KH, ldq, ldk, ldv, ldo, scale, window, softcap);
     }
   } else {
@@ -832,28 +868,9 @@ extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void*
   const float scale = 1.f / sqrtf((float)D);
   const bf16 *qp = (const bf16*)q, *kp = (const bf16*)k, *vp = (const bf16*)v, *op = (const bf16*)o, *gop = (const bf16*)d_o;
   float* delta = (float*)workspace;
-  const bool fast = fast_ok(D, q, k, v, o, ldq, ldk, ldv, ldo) && aligned16(d_o) && aligned16(dq) && aligned16(dk) && aligned16(dv) &&
-                    lddo % 8 == 0 && lddq % 8 == 0 && lddk % 8 == 0 && lddv % 8 == 0;
-  if (fast) {
-    const int64_t units = (int64_t)B * S * H;
-    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((units + 15) / 16)), dim3(256), 0, stream, op, gop, delta, B, S, H, ldo, lddo);
-    dim3 gkv((unsigned)(((S + 127) / 128) * KH * B)), gq((unsigned)(((S + 127) / 128) * H * B));
-    constexpr int SM_KV = 2 * (2 * 32 * 256 + 256) + 128 * 256;
-    static bool set = false;
-    if (!set) {
-      (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
-      (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
-      (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-      (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-      set = true;
-    }
-    if (softcap > 0.f) {
-      hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, gkv, dim3(256), SM_KV, stream, qp, kp, vp, gop, lse, delta, (bf16*)dk, (bf16*)dv, S, H, KH, ldq, ldk, ldv, lddo, lddk, lddv, scale, window, softcap);
-      hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, gq, dim3(256), 65536, stream, qp, kp, vp, gop, lse, delta, (bf16*)dq, S, H, KH, ldq, ldk, ldv, lddo, lddq, scale, window, softcap);
-    } else {
-      hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, gkv, dim3(256), SM_KV, stream, qp, kp, vp, gop, lse, delta, (bf16*)dk, (bf16*)dv, S, H, KH, ldq, ldk, ldv, lddo, lddk, lddv, scale, window, softcap);
-      hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, gq, dim3(256), 65536, stream, qp, kp, vp, gop, lse, delta, (bf16*)dq, S, H, KH, ldq, ldk, ldv, lddo, lddq, scale, window, softcap);
-    }
+  if (bwd_fast_ok(q, k, v, o, d_o, dq, dk, dv, D, ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv)) {
+    launch_bwd_fast(stream, qp, kp, vp, op, lse, gop, (bf16*)dq, (bf16*)dk, (bf16*)dv, delta, B, S, H, KH, ldq, ldk, ldv, ldo, lddo,
+                    lddq, lddk, lddv, window, softcap);
   } else {
     OLMAX_CHECK(D <= 256 && (size_t)S * 8 <= 65536, OLMAX_ERR_SHAPE, "olmax_attn_bwd: generic path supports head_dim <= 256 and seq_len <= 8192");
     const int64_t accb = attn_acc_bytes(B, S, KH, D);
