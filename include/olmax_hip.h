@@ -138,6 +138,22 @@ int32_t olmax_attn_bwd(olmax_stream_t stream, const void* q, const void* k, cons
                        int64_t lddo, int64_t lddq, int64_t lddk, int64_t lddv, int32_t window,
                        float softcap);
 
+/* olmax_attn_bwd without a workspace argument.  No counterpart in the reference: it exists for
+ * callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  The delta scratch ([B, H, S] fp32) lives in a device array
+ * inside the library (4 MiB per GPU, held until the process ends): batch*heads*seq_len must not
+ * exceed olmax_attn_bwd_noalloc_max_rows() (2^20), head_dim must be 128 and every pointer 16-byte
+ * aligned with row strides that are multiples of 8, otherwise an error is returned and nothing
+ * is launched.  Calls no hipMalloc / hipFree.  All calls on one GPU share the array: calls that
+ * overlap on one GPU (different streams or threads) race.  Results equal olmax_attn_bwd's bit for
+ * bit (same kernels). */
+int64_t olmax_attn_bwd_noalloc_max_rows(void);
+int32_t olmax_attn_bwd_noalloc(olmax_stream_t stream, const void* q, const void* k, const void* v,
+                               const void* o, const float* lse, const void* d_o, void* dq, void* dk,
+                               void* dv, int32_t B, int32_t S, int32_t H, int32_t KH, int32_t D,
+                               int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
+                               int64_t lddq, int64_t lddk, int64_t lddv, int32_t window, float softcap);
+
 /* ---- Cross entropy: cross_entropy_loss / fused_cross_entropy_loss,
  * src/olmax/nn/functional.py:70-121 (reduction "mean"; see the label quirks there).
  * logits bf16 (logits_f32 == 0) or fp32; dlogits (optional, may alias logits) receives

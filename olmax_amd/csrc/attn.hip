@@ -888,3 +888,61 @@ extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void*
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
 }
+
+// ---------------------------------------------------------------------------------------
+// olmax_attn_bwd for callers that cannot allocate (code under HIP graph capture, serving loops,
+// harnesses that forbid hipMalloc): the delta scratch lives in a file-scope device array
+// instead of a caller-provided workspace.  Each GPU the library runs on holds its own copy of the
+// array (4 MiB) until the process ends; every call on a GPU shares it, so calls that overlap on
+// one GPU (two streams, two threads) race on it.  Nothing in it has to start at zero: the first
+// kernel of a call writes every delta entry the other two read.
+// ---------------------------------------------------------------------------------------
+constexpr int64_t ATTN_SCRATCH_FLOATS = 1 << 20;  // B * H * S <= 1 Mi (4 MiB)
+static __device__ __align__(256) float scratch[ATTN_SCRATCH_FLOATS];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[MAX_DEVICES];  // device address of `scratch` on each GPU, resolved on first use
+
+// The array's name is only a host-side handle; its device address differs per GPU and comes
+// from hipGetSymbolAddress with that GPU current.
+int scratch_for_current_device(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+    return olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_attn_bwd_noalloc: cannot identify the current device");
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    float* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_attn_bwd_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return OLMAX_OK;
+}
+}  // namespace
+
+extern "C" int64_t olmax_attn_bwd_noalloc_max_rows(void) { return ATTN_SCRATCH_FLOATS; }
+
+extern "C" int32_t olmax_attn_bwd_noalloc(hipStream_t stream, const void* q, const void* k, const void* v,
+                                          const void* o, const float* lse, const void* d_o, void* dq, void* dk,
+                                          void* dv, int32_t B, int32_t S, int32_t H, int32_t KH, int32_t D,
+                                          int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
+                                          int64_t lddq, int64_t lddk, int64_t lddv, int32_t window, float softcap) {
+  OLMAX_CHECK(q && k && v && o && lse && d_o && dq && dk && dv, OLMAX_ERR_ARG, "olmax_attn_bwd_noalloc: null pointer");
+  OLMAX_CHECK(B > 0 && S > 0 && H > 0 && KH > 0 && D > 0 && H % KH == 0, OLMAX_ERR_SHAPE, "olmax_attn_bwd_noalloc: bad shape");
+  OLMAX_CHECK(ldq >= (int64_t)H * D && ldo >= (int64_t)H * D && lddo >= (int64_t)H * D && lddq >= (int64_t)H * D && ldk >= (int64_t)KH * D && ldv >= (int64_t)KH * D && lddk >= (int64_t)KH * D && lddv >= (int64_t)KH * D, OLMAX_ERR_SHAPE, "olmax_attn_bwd_noalloc: row stride smaller than heads*head_dim");
+  OLMAX_CHECK((int64_t)B * H * S <= ATTN_SCRATCH_FLOATS, OLMAX_ERR_WORKSPACE,
+              "olmax_attn_bwd_noalloc: batch*heads*seq_len = %ld exceeds the built-in scratch of %ld rows; use olmax_attn_bwd with a workspace",
+              (long)((int64_t)B * H * S), (long)ATTN_SCRATCH_FLOATS);
+  OLMAX_CHECK(bwd_fast_ok(q, k, v, o, d_o, dq, dk, dv, D, ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv), OLMAX_ERR_ALIGN,
+              "olmax_attn_bwd_noalloc: needs head_dim 128, 16-byte aligned pointers and row strides that are multiples of 8; use olmax_attn_bwd otherwise");
+  float* delta = nullptr;
+  { int rc = scratch_for_current_device(&delta); if (rc) return rc; }
+  launch_bwd_fast(stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)o, lse, (const bf16*)d_o, (bf16*)dq, (bf16*)dk,
+                  (bf16*)dv, delta, B, S, H, KH, ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv, window, softcap);
+  OLMAX_LAUNCH_CHECK();
+  return OLMAX_OK;
+}
