@@ -226,7 +226,9 @@ typedef struct {
   int32_t layer_type; /* 0 TransformerLayer (pre-norm, layer.py:80-94), 1 ReorderedNorm
                          (layer.py:102-116), 2 Gemma pre+post (layer.py:169-185) */
   int32_t act;        /* 0 silu, 1 gelu-tanh */
-  int32_t qk_norm;    /* head-wise QK-norm (attention.py:293-296) */
+  int32_t qk_norm;    /* 0 off; 1 head-wise QK-norm, weight [head_dim] shared by the heads
+                         (attention.py:293-296); 2 full width, weights [n_heads*head_dim] for q and
+                         [n_kv_heads*head_dim] for k, before the reshape (attention.py:281-284) */
   int32_t tied;       /* LM head shares the embedding matrix (extension) */
   int32_t batch, seq_len;
   int32_t checkpoint; /* 1: full-block activation checkpointing (NothingSaveable,
@@ -278,14 +280,16 @@ int32_t olmax_model_loss(olmax_stream_t stream, const olmax_model_config* cfg, c
                          float* loss, void* workspace, int64_t workspace_bytes);
 
 /* step_optimizer, src/olmax/train/trainer.py:742-757: fused AdamW over every leaf.
- * decay_embedding == 0 masks "embedding.weight" from weight decay as the benchmark does
- * (src/integration_tests/train_transformer.py:388).  max_grad_norm > 0 applies
+ * leaf_decay: host array with one entry per leaf in olmax_model_layout order, 0 = the leaf is
+ * exempt from weight decay, the mask of OptimConfig.build_weight_decay_mask
+ * (src/olmax/optim/config.py:94-122; the benchmark exempts "embedding.weight",
+ * src/integration_tests/train_transformer.py:388); NULL = every leaf decays.  max_grad_norm > 0 applies
  * clip_grads_by_global_norm (src/olmax/optim/utils.py:22-38); norm_scratch: device float[2], left holding
  * {clip factor, gradient norm}. */
 int32_t olmax_model_adamw(olmax_stream_t stream, const olmax_model_config* cfg, float* master,
                           float* m, float* v, void* params_bf16, const void* grad_bf16,
                           const float* grad_f32, int64_t step, float lr, float b1, float b2, float eps,
-                          float wd, int32_t decay_embedding, float max_grad_norm, float* norm_scratch);
+                          float wd, const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch);
 
 /* Gradient accumulation over micro-batches: optax.MultiSteps as built at
  * src/olmax/optim/config.py:153-154 and driven once per micro-batch by train_batch,
@@ -301,7 +305,7 @@ int32_t olmax_model_grad_accumulate(olmax_stream_t stream, const olmax_model_con
 int32_t olmax_model_adamw_accumulated(olmax_stream_t stream, const olmax_model_config* cfg, float* master,
                                       float* m, float* v, void* params_bf16, const float* acc, int64_t step,
                                       float lr, float b1, float b2, float eps, float wd,
-                                      int32_t decay_embedding, float max_grad_norm, float* norm_scratch);
+                                      const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch);
 
 /* process_microbatch, src/olmax/train/trainer.py:759-777: loss + gradients + AdamW in one call.
  * opt_stream (optional, default priority, != stream): when given, clipping is off and the config
@@ -314,7 +318,7 @@ int32_t olmax_model_train_step(olmax_stream_t stream, olmax_stream_t opt_stream,
                                void* params_bf16, const int32_t* ids, const int32_t* labels, float* loss,
                                void* grad_bf16, float* grad_f32, void* workspace, int64_t workspace_bytes,
                                int64_t step, float lr, float b1, float b2, float eps, float wd,
-                               int32_t decay_embedding, float max_grad_norm, float* norm_scratch);
+                               const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch);
 
 /* Single transformer block in isolation (any of the three orderings). */
 typedef struct {

@@ -15,7 +15,7 @@ int olmax_set_error(int code, const char* fmt, ...) {
 
 extern "C" const char* olmax_last_error_string(void) { return g_err; }
 
-extern "C" int32_t olmax_abi_version(void) { return 1; }
+extern "C" int32_t olmax_abi_version(void) { return 2; }
 
 // ---- profiler ranges.  The reference wraps its modules in jax.named_scope / starts a JAX trace
 // from ProfilerCallback (src/olmax/train/callbacks/profiler.py:33-50); here the whole-model entry

@@ -40,6 +40,7 @@ int check_cfg(const olmax_model_config* c) {
               OLMAX_ERR_SHAPE, "model config: sizes must be positive");
   OLMAX_CHECK(c->n_heads % c->n_kv_heads == 0, OLMAX_ERR_SHAPE, "model config: n_heads must be a multiple of n_kv_heads");
   OLMAX_CHECK(c->layer_type >= 0 && c->layer_type <= 2 && (c->act == 0 || c->act == 1), OLMAX_ERR_ARG, "model config: bad layer_type/act");
+  OLMAX_CHECK(c->qk_norm >= 0 && c->qk_norm <= 2, OLMAX_ERR_ARG, "model config: qk_norm must be 0 (off), 1 (head-wise) or 2 (full width)");
   OLMAX_CHECK(c->head_dim % 2 == 0, OLMAX_ERR_SHAPE, "model config: head_dim must be even");
   OLMAX_CHECK(c->d_model % 8 == 0 && c->hidden % 8 == 0 && c->head_dim % 8 == 0, OLMAX_ERR_SHAPE,
               "model config: d_model, hidden and head_dim must be multiples of 8 (128-bit rows)");
@@ -154,7 +155,16 @@ int block_forward(hipStream_t s, const olmax_model_config* c, const olmax_block_
     RC(lin_fwd(s, attn_in, m.d, w->wqkv, m.d, m.QKV, a.qkv, m.QKV, nullptr, 0, m.T));
   const bf16 *qp, *kp;
   int64_t ldqk;
-  if (c->qk_norm) {
+  if (c->qk_norm == 2) {
+    // full-width QK-norm (attention.py:281-284): one RMSNorm over all heads of q (and of k)
+    // before the reshape, then the rotation of the normalised heads in place
+    ldqk = m.HD + m.KD;
+    RC(olmax_rmsnorm_fwd(s, a.qkv, w->q_norm, a.qkr, m.T, m.HD, m.QKV, ldqk, eps));
+    RC(olmax_rmsnorm_fwd(s, a.qkv + m.HD, w->k_norm, a.qkr + m.HD, m.T, m.KD, m.QKV, ldqk, eps));
+    RC(olmax_qk_rope_fwd(s, a.qkr, a.qkr, nullptr, cos_t, sin_t, m.T, m.H + m.K, m.D, m.S, ldqk, ldqk, eps));
+    qp = a.qkr;
+    kp = a.qkr + m.HD;
+  } else if (c->qk_norm) {
     ldqk = m.HD + m.KD;
     RC(olmax_qk_rope_fwd(s, a.qkv, a.qkr, w->q_norm, cos_t, sin_t, m.T, m.H, m.D, m.S, m.QKV, ldqk, eps));
     RC(olmax_qk_rope_fwd(s, a.qkv + m.HD, a.qkr + m.HD, w->k_norm, cos_t, sin_t, m.T, m.K, m.D, m.S, m.QKV, ldqk, eps));
@@ -212,10 +222,17 @@ int attn_backward(hipStream_t s, const olmax_model_config* c, const olmax_block_
     RC(olmax_attn_bwd(s, a.qkr, a.qkr + m.HD, vp, a.o, a.lse, t.d_o, t.dqkr, t.dqkr + m.HD, t.dqkv + m.HD + m.KD,
                       t.attn_ws, t.attn_ws_bytes, m.B, m.S, m.H, m.K, m.D, ldqk, ldqk, m.QKV, m.HD, m.HD, ldqk, ldqk,
                       m.QKV, window, c->attn_softcap));
-    RC(olmax_qk_rope_bwd(s, t.dqkr, t.dqkv, a.qkv, w->q_norm, g->q_norm, cos_t, sin_t, m.T, m.H, m.D, m.S, ldqk, m.QKV,
-                         m.QKV, eps));
-    RC(olmax_qk_rope_bwd(s, t.dqkr + m.HD, t.dqkv + m.HD, a.qkv + m.HD, w->k_norm, g->k_norm, cos_t, sin_t, m.T, m.K,
-                         m.D, m.S, ldqk, m.QKV, m.QKV, eps));
+    if (c->qk_norm == 2) {
+      RC(olmax_qk_rope_bwd(s, t.dqkr, t.dqkr, nullptr, nullptr, nullptr, cos_t, sin_t, m.T, m.H + m.K, m.D, m.S, ldqk, ldqk, 0, eps));
+      RC(olmax_rmsnorm_bwd(s, a.qkv, w->q_norm, t.dqkr, nullptr, t.dqkv, g->q_norm, m.T, m.HD, m.QKV, ldqk, 0, m.QKV, eps));
+      RC(olmax_rmsnorm_bwd(s, a.qkv + m.HD, w->k_norm, t.dqkr + m.HD, nullptr, t.dqkv + m.HD, g->k_norm, m.T, m.KD, m.QKV, ldqk, 0,
+                           m.QKV, eps));
+    } else {
+      RC(olmax_qk_rope_bwd(s, t.dqkr, t.dqkv, a.qkv, w->q_norm, g->q_norm, cos_t, sin_t, m.T, m.H, m.D, m.S, ldqk, m.QKV,
+                           m.QKV, eps));
+      RC(olmax_qk_rope_bwd(s, t.dqkr + m.HD, t.dqkv + m.HD, a.qkv + m.HD, w->k_norm, g->k_norm, cos_t, sin_t, m.T, m.K,
+                           m.D, m.S, ldqk, m.QKV, m.QKV, eps));
+    }
   } else {
     RC(olmax_attn_bwd(s, a.qkv, a.qkv + m.HD, vp, a.o, a.lse, t.d_o, t.dqkv, t.dqkv + m.HD, t.dqkv + m.HD + m.KD,
                       t.attn_ws, t.attn_ws_bytes, m.B, m.S, m.H, m.K, m.D, m.QKV, m.QKV, m.QKV, m.HD, m.HD, m.QKV,
@@ -295,26 +312,27 @@ void layer_offsets(const olmax_model_config* c, int l, const Layout& L, int64_t 
   o.mlp_norm = p; p += m.d;
   o.attn_in_norm = o.mlp_in_norm = o.q_norm = o.k_norm = -1;
   if (c->layer_type == 2) { o.attn_in_norm = p; p += m.d; o.mlp_in_norm = p; p += m.d; }
-  if (c->qk_norm) { o.q_norm = p; p += m.D; o.k_norm = p; p += m.D; }
+  const int qn = c->qk_norm == 2 ? m.HD : m.D, kn = c->qk_norm == 2 ? m.KD : m.D;  // full width or per head
+  if (c->qk_norm) { o.q_norm = p; p += qn; o.k_norm = p; p += kn; }
   int64_t f = L.f_embedding + (int64_t)c->vocab * m.d + (int64_t)l * per_layer_f;
   o.f_attn_norm = f; f += m.d;
   o.f_mlp_norm = f; f += m.d;
   o.f_attn_in_norm = o.f_mlp_in_norm = o.f_q_norm = o.f_k_norm = -1;
   if (c->layer_type == 2) { o.f_attn_in_norm = f; f += m.d; o.f_mlp_in_norm = f; f += m.d; }
-  if (c->qk_norm) { o.f_q_norm = f; f += m.D; o.f_k_norm = f; f += m.D; }
+  if (c->qk_norm) { o.f_q_norm = f; f += qn; o.f_k_norm = f; f += kn; }
 }
 int64_t per_layer_params(const olmax_model_config* c) {
   const Dims m = dims_of(c);
   int64_t n = (int64_t)m.QKV * m.d + (int64_t)m.d * m.HD + (int64_t)3 * m.F * m.d + 2 * m.d;
   if (c->layer_type == 2) n += 2 * m.d;
-  if (c->qk_norm) n += 2 * m.D;
+  if (c->qk_norm) n += c->qk_norm == 2 ? m.HD + m.KD : 2 * m.D;
   return n;
 }
 int64_t per_layer_f32(const olmax_model_config* c) {
   const Dims m = dims_of(c);
   int64_t n = 2 * m.d;
   if (c->layer_type == 2) n += 2 * m.d;
-  if (c->qk_norm) n += 2 * m.D;
+  if (c->qk_norm) n += c->qk_norm == 2 ? m.HD + m.KD : 2 * m.D;
   return n;
 }
 Layout layout_of(const olmax_model_config* c) {
@@ -489,14 +507,16 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
 }
 
 // AdamW over the leaves [begin, end) of a layout; runs of adjacent bf16-gradient leaves with
-// the same decay become single launches.
+// the same decay become single launches.  leaf_decay (host, one entry per leaf of the layout;
+// NULL: every leaf decays) is the weight-decay mask of AdamWConfig.build.
 int adamw_leaves(hipStream_t s, const olmax_leaf* leaves, int begin, int end, float* master, float* mom, float* var,
                  bf16* shadow, const bf16* G, const float* grad_f32, int64_t step, float lr, float b1, float b2,
-                 float eps, float wd, int decay_embedding, const float* dscale, int grid_cap = 512) {
+                 float eps, float wd, const int32_t* leaf_decay, const float* dscale, int grid_cap = 512) {
+  auto decays = [&](int i) { return !leaf_decay || leaf_decay[i] != 0; };
   int i = begin;
   while (i < end) {
     const olmax_leaf& lf = leaves[i];
-    const float lwd = (lf.kind == OLMAX_LEAF_EMBEDDING && !decay_embedding) ? 0.f : wd;
+    const float lwd = decays(i) ? wd : 0.f;
     if (lf.grad_f32) {
       RC(olmax_adamw_grid(s, master + lf.offset, grad_f32 + lf.grad_f32_offset, mom + lf.offset, var + lf.offset,
                           shadow + lf.offset, lf.numel, 0, lr, b1, b2, eps, lwd, step, 1.f, dscale, grid_cap));
@@ -504,7 +524,7 @@ int adamw_leaves(hipStream_t s, const olmax_leaf* leaves, int begin, int end, fl
     } else {
       int64_t n = lf.numel;
       int j = i + 1;
-      while (j < end && !leaves[j].grad_f32 && leaves[j].offset == lf.offset + n) {
+      while (j < end && !leaves[j].grad_f32 && leaves[j].offset == lf.offset + n && decays(j) == decays(i)) {
         n += leaves[j].numel;
         j++;
       }
@@ -529,7 +549,7 @@ struct OverlapCtx {
   const float* grad_f32;
   int64_t step;
   float lr, b1, b2, eps, wd;
-  int decay_embedding;
+  const int32_t* leaf_decay;
   // 0: launch as soon as the gradients are final; else at that StepHook point.  Measured on
   // the 7B step: AdamW as a one-workgroup-per-CU grid of 32-register waves launched at once
   // (it then shares CUs with the next block's forward GEMMs, whose waves leave it 32 registers
@@ -570,7 +590,7 @@ int overlap_launch(OverlapCtx* x, int layer) {
   if (hipEventRecord(x->ev, x->main) != hipSuccess || hipStreamWaitEvent(x->opt, x->ev, 0) != hipSuccess)
     return olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_model_train_step: event record/wait failed");
   return adamw_leaves(x->opt, x->leaves, begin, end, x->master, x->mom, x->var, x->shadow, x->G, x->grad_f32, x->step, x->lr,
-                      x->b1, x->b2, x->eps, x->wd, x->decay_embedding, nullptr, 256);
+                      x->b1, x->b2, x->eps, x->wd, x->leaf_decay, nullptr, 256);
 }
 
 __global__ void clip_scale_kernel(const float* sumsq, float max_norm, float* out) {
@@ -622,8 +642,8 @@ extern "C" int32_t olmax_model_layout(const olmax_model_config* c, olmax_leaf* o
       put(OLMAX_LEAF_MLP_IN_NORM, l, o.mlp_in_norm, 1, m.d, 1, o.f_mlp_in_norm);
     }
     if (c->qk_norm) {
-      put(OLMAX_LEAF_Q_NORM, l, o.q_norm, 1, m.D, 1, o.f_q_norm);
-      put(OLMAX_LEAF_K_NORM, l, o.k_norm, 1, m.D, 1, o.f_k_norm);
+      put(OLMAX_LEAF_Q_NORM, l, o.q_norm, 1, c->qk_norm == 2 ? m.HD : m.D, 1, o.f_q_norm);
+      put(OLMAX_LEAF_K_NORM, l, o.k_norm, 1, c->qk_norm == 2 ? m.KD : m.D, 1, o.f_k_norm);
     }
   }
   put(OLMAX_LEAF_FINAL_NORM, -1, L.final_norm, 1, m.d, 1, L.f_final_norm);
@@ -696,7 +716,7 @@ extern "C" int32_t olmax_model_loss(hipStream_t s, const olmax_model_config* c, 
 
 extern "C" int32_t olmax_model_adamw(hipStream_t s, const olmax_model_config* c, float* master, float* mom, float* var,
                                      void* params_bf16, const void* grad_bf16, const float* grad_f32, int64_t step,
-                                     float lr, float b1, float b2, float eps, float wd, int32_t decay_embedding,
+                                     float lr, float b1, float b2, float eps, float wd, const int32_t* leaf_decay,
                                      float max_grad_norm, float* norm_scratch) {
   RC(check_cfg(c));
   OLMAX_CHECK(master && mom && var && params_bf16 && grad_bf16 && grad_f32, OLMAX_ERR_ARG, "olmax_model_adamw: null pointer");
@@ -722,7 +742,7 @@ extern "C" int32_t olmax_model_adamw(hipStream_t s, const olmax_model_config* c,
       dscale = norm_scratch;
     }
   }
-  if (!rc) rc = adamw_leaves(s, leaves, 0, nleaf, master, mom, var, shadow, G, grad_f32, step, lr, b1, b2, eps, wd, decay_embedding, dscale);
+  if (!rc) rc = adamw_leaves(s, leaves, 0, nleaf, master, mom, var, shadow, G, grad_f32, step, lr, b1, b2, eps, wd, leaf_decay, dscale);
   delete[] leaves;
   return rc;
 }
@@ -762,7 +782,7 @@ extern "C" int32_t olmax_model_grad_accumulate(hipStream_t s, const olmax_model_
 // reference chains it inside MultiSteps.
 extern "C" int32_t olmax_model_adamw_accumulated(hipStream_t s, const olmax_model_config* c, float* master, float* mom,
                                                  float* var, void* params_bf16, const float* acc, int64_t step, float lr,
-                                                 float b1, float b2, float eps, float wd, int32_t decay_embedding,
+                                                 float b1, float b2, float eps, float wd, const int32_t* leaf_decay,
                                                  float max_grad_norm, float* norm_scratch) {
   RC(check_cfg(c));
   OLMAX_CHECK(master && mom && var && params_bf16 && acc, OLMAX_ERR_ARG, "olmax_model_adamw_accumulated: null pointer");
@@ -777,11 +797,23 @@ extern "C" int32_t olmax_model_adamw_accumulated(hipStream_t s, const olmax_mode
     hipLaunchKernelGGL(clip_scale_kernel, dim3(1), dim3(1), 0, s, norm_scratch, max_grad_norm, norm_scratch);
     dscale = norm_scratch;
   }
-  // the embedding (first in the layout) may be exempt from weight decay; everything else decays
-  const int64_t ne = L.layers_begin;
-  RC(olmax_adamw_dscale(s, master, acc, mom, var, shadow, ne, 0, lr, b1, b2, eps, decay_embedding ? wd : 0.f, step, 1.f, dscale));
-  return olmax_adamw_dscale(s, master + ne, acc + ne, mom + ne, var + ne, shadow + ne, L.total - ne, 0, lr, b1, b2, eps, wd,
-                            step, 1.f, dscale);
+  // the leaves tile the flat buffers in layout order: one launch per run of leaves with the same decay
+  const int nleaf = olmax_model_layout(c, nullptr, 0);
+  olmax_leaf* leaves = new olmax_leaf[nleaf];
+  olmax_model_layout(c, leaves, nleaf);
+  auto decays = [&](int i) { return !leaf_decay || leaf_decay[i] != 0; };
+  int rc = OLMAX_OK;
+  for (int i = 0; i < nleaf && !rc;) {
+    int j = i + 1;
+    int64_t n = leaves[i].numel;
+    while (j < nleaf && decays(j) == decays(i) && leaves[j].offset == leaves[i].offset + n) n += leaves[j++].numel;
+    const int64_t o = leaves[i].offset;
+    rc = olmax_adamw_dscale(s, master + o, acc + o, mom + o, var + o, shadow + o, n, 0, lr, b1, b2, eps, decays(i) ? wd : 0.f, step,
+                            1.f, dscale);
+    i = j;
+  }
+  delete[] leaves;
+  return rc;
 }
 
 // One micro-batch of training: loss + gradients, then AdamW.  With a second stream and no
@@ -795,7 +827,7 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
                                           void* params_bf16, const int32_t* ids, const int32_t* labels, float* loss,
                                           void* grad_bf16, float* grad_f32, void* workspace, int64_t workspace_bytes,
                                           int64_t step, float lr, float b1, float b2, float eps, float wd,
-                                          int32_t decay_embedding, float max_grad_norm, float* norm_scratch) {
+                                          const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch) {
   RC(check_cfg(c));
   OLMAX_CHECK(master && mom && var && params_bf16 && grad_bf16 && grad_f32, OLMAX_ERR_ARG, "olmax_model_train_step: null pointer");
   OLMAX_CHECK(step >= 1, OLMAX_ERR_ARG, "olmax_model_train_step: step is 1-based");
@@ -805,7 +837,7 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
     RC(model_run(stream, c, windows, cos_tables, sin_tables, params_bf16, ids, labels, loss, grad_bf16, grad_f32, workspace,
                  workspace_bytes, true));
     return olmax_model_adamw(stream, c, master, mom, var, params_bf16, grad_bf16, grad_f32, step, lr, b1, b2, eps, wd,
-                             decay_embedding, max_grad_norm, norm_scratch);
+                             leaf_decay, max_grad_norm, norm_scratch);
   }
   // one event per thread, created on first use and kept for the life of the process
   static thread_local hipEvent_t ev = nullptr;
@@ -815,7 +847,7 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
   olmax_leaf* leaves = new olmax_leaf[nleaf];
   olmax_model_layout(c, leaves, nleaf);
   OverlapCtx x{stream, opt_stream, ev, leaves, nleaf, master, mom, var, (bf16*)params_bf16, (const bf16*)grad_bf16, grad_f32,
-               step, lr, b1, b2, eps, wd, decay_embedding, 0, {0, 0, 0, 0}, 0};
+               step, lr, b1, b2, eps, wd, leaf_decay, 0, {0, 0, 0, 0}, 0};
   // the optimizer stream must not run ahead of work already queued on the main stream
   int rc = OLMAX_OK;
   if (hipEventRecord(ev, stream) != hipSuccess || hipStreamWaitEvent(opt_stream, ev, 0) != hipSuccess)

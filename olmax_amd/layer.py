@@ -41,9 +41,9 @@ class TransformerBlock:
         if c.layer_type == "gemma":
             self.norms["attention_input_norm"] = torch.ones(d, device=dev, dtype=BF16)
             self.norms["mlp_input_norm"] = torch.ones(d, device=dev, dtype=BF16)
-        if c.qk_norm_headwise:
-            self.norms["attention.q_norm"] = torch.ones(D, device=dev, dtype=BF16)
-            self.norms["attention.k_norm"] = torch.ones(D, device=dev, dtype=BF16)
+        if c.qk_norm:  # head-wise: one weight [D]; full width: [H*D] for q, [K*D] for k
+            self.norms["attention.q_norm"] = torch.ones(D if c.qk_norm_headwise else H * D, device=dev, dtype=BF16)
+            self.norms["attention.k_norm"] = torch.ones(D if c.qk_norm_headwise else K * D, device=dev, dtype=BF16)
         self.window = c.windows()[layer_idx] if c.num_layers > layer_idx else (-1 if c.window_size is None else c.window_size)
         theta = c.thetas()[layer_idx] if c.num_layers > layer_idx else c.rope_theta
         self.cos, self.sin = ops.rope_tables(sequence_length, D, theta, dev)

@@ -55,8 +55,8 @@ class WarmupStableDecaySchedule:
 @dataclass
 class AdamWConfig:
     """src/olmax/optim/config.py:125-156.  ``no_decay_modules`` are fnmatch patterns over the
-    dotted leaf paths; the fused step supports masking ``embedding.weight`` (what the benchmark
-    uses, src/integration_tests/train_transformer.py:388)."""
+    dotted leaf paths (build_weight_decay_mask, config.py:94-122); the benchmark masks
+    ``embedding.weight`` (src/integration_tests/train_transformer.py:388)."""
     lr: object = field(default_factory=lambda: ConstantSchedule(1e-4))
     b1: float = 0.9
     b2: float = 0.999
@@ -65,12 +65,9 @@ class AdamWConfig:
     no_decay_modules: Optional[List[str]] = None
     max_grad_norm: Optional[float] = None
 
-    def decay_embedding(self) -> bool:
-        pats = self.no_decay_modules or []
-        for p in pats:
-            if not fnmatch.fnmatch("embedding.weight", p):
-                raise NotImplementedError(f"no_decay pattern {p!r}: only 'embedding.weight' can be masked in the fused step")
-        return not any(fnmatch.fnmatch("embedding.weight", p) for p in pats)
+    def decays(self, name: str) -> bool:
+        """Whether the leaf with this dotted path takes weight decay."""
+        return not any(fnmatch.fnmatch(name, p) for p in (self.no_decay_modules or []))
 
     def lr_at(self, count: int) -> float:
         """Learning rate read at the pre-increment count (first step uses schedule(0))."""

@@ -82,7 +82,8 @@ class Trainer:
         self.model, self.optim = model, optim
         self.overlap_optimizer = overlap_optimizer
         self.count = 0  # optimizer steps taken
-        self._decay_embedding = optim.decay_embedding()
+        self._no_decay = tuple(optim.no_decay_modules or ())
+        model.weight_decay_mask(self._no_decay)  # warns now about patterns that match nothing
         model.init_optimizer_state()
 
     def process_microbatch(self, input_ids: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
@@ -90,7 +91,7 @@ class Trainer:
         self.count += 1
         return self.model.train_step(input_ids, labels, step=self.count, lr=lr, b1=self.optim.b1, b2=self.optim.b2,
                                      eps=self.optim.eps, weight_decay=self.optim.weight_decay,
-                                     decay_embedding=self._decay_embedding, max_grad_norm=self.optim.max_grad_norm,
+                                     no_decay_modules=self._no_decay, max_grad_norm=self.optim.max_grad_norm,
                                      overlap_optimizer=self.overlap_optimizer)
 
     def train_batch(self, batch: Sequence[Tuple[torch.Tensor, torch.Tensor]]) -> torch.Tensor:
@@ -112,7 +113,7 @@ class Trainer:
             losses.append(self.model.loss_and_grads(ids, labels).clone())
             self.model.accumulate_grads(j)
         self.model.adamw_step_accumulated(step=self.count, lr=lr, b1=self.optim.b1, b2=self.optim.b2, eps=self.optim.eps,
-                                          weight_decay=self.optim.weight_decay, decay_embedding=self._decay_embedding,
+                                          weight_decay=self.optim.weight_decay, no_decay_modules=self._no_decay,
                                           max_grad_norm=self.optim.max_grad_norm)
         return torch.stack(losses).mean()
 
@@ -160,8 +161,11 @@ class Trainer:
         meter = ThroughputMeter()
         step_this_run = 0
         t0 = time.perf_counter()
-        for batch in data_loader:
-            if self.count >= max_steps:
+        batches = iter(data_loader)
+        while self.count < max_steps:  # tested BEFORE the next batch is pulled (trainer.py:522-551):
+            try:                       # the loader state stays at what was trained on
+                batch = next(batches)
+            except StopIteration:
                 break
             step_this_run += 1
             tokens = tokens_per_batch if tokens_per_batch is not None else sum(int(ids.numel()) for ids, _ in batch)

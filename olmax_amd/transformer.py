@@ -70,7 +70,9 @@ class TransformerConfig:
     head_dim: Optional[int] = None
     layer_type: str = "default"            # "default" | "reordered_norm" | "gemma"
     activation: str = "silu"               # "silu" | "gelu" (tanh approximation)
-    qk_norm_headwise: bool = False
+    qk_norm_headwise: bool = False         # QK-norm with one weight [head_dim] shared by the heads (attention.py:293-296)
+    qk_norm: Optional[bool] = None         # None: on iff qk_norm_headwise; True with qk_norm_headwise False:
+                                           # full-width QK-norm before the reshape (attention.py:281-284)
     norm_eps: float = 1e-5                 # RMSNormConfig default, normalization.py:95
     rope_theta: float = 10_000.0
     rope_theta_per_layer: Optional[Sequence[float]] = None
@@ -90,6 +92,10 @@ class TransformerConfig:
             raise ValueError(f"unknown layer_type {self.layer_type!r}")
         if self.activation not in ACTIVATIONS:
             raise ValueError(f"unknown activation {self.activation!r}")
+        if self.qk_norm is None:
+            self.qk_norm = self.qk_norm_headwise
+        if self.qk_norm_headwise and not self.qk_norm:
+            raise ValueError("qk_norm_headwise needs qk_norm")
         if self.layer_ac_policy not in (None, "nothing_saveable"):
             raise ValueError("layer_ac_policy must be None or 'nothing_saveable' (full block)")
 
@@ -98,6 +104,10 @@ class TransformerConfig:
             assert len(self.window_size_per_layer) == self.num_layers
             return [-1 if w is None else int(w) for w in self.window_size_per_layer]
         return [-1 if self.window_size is None else int(self.window_size)] * self.num_layers
+
+    def qk_norm_mode(self) -> int:
+        """0 off, 1 head-wise, 2 full width (olmax_model_config.qk_norm)."""
+        return 0 if not self.qk_norm else (1 if self.qk_norm_headwise else 2)
 
     def thetas(self) -> List[float]:
         if self.rope_theta_per_layer is not None:
@@ -110,7 +120,7 @@ class TransformerConfig:
             vocab=self.vocab_size, d_model=self.d_model, n_layers=self.num_layers, n_heads=self.n_heads,
             n_kv_heads=self.n_kv_heads, head_dim=self.head_dim, hidden=self.hidden_size,
             layer_type=LAYER_TYPES[self.layer_type], act=ACTIVATIONS[self.activation],
-            qk_norm=int(self.qk_norm_headwise), tied=int(self.tie_embeddings), batch=batch, seq_len=seq_len,
+            qk_norm=self.qk_norm_mode(), tied=int(self.tie_embeddings), batch=batch, seq_len=seq_len,
             checkpoint=int(self.layer_ac_policy == "nothing_saveable"), eps=self.norm_eps,
             attn_softcap=self.attn_logit_softcap, final_softcap=self.final_logit_softcap)
 
@@ -232,6 +242,7 @@ class Transformer:
         self.grad_acc = None  # fp32 running mean over micro-batches, allocated on first use
         self._workspace: Optional[torch.Tensor] = None
         self._opt_stream = None
+        self._decay_masks: Dict[tuple, object] = {}
 
         # per-layer windows and RoPE tables (get_buffer_cache, model.py:138-144)
         self._windows = (ctypes.c_int32 * max(1, config.num_layers))(*config.windows())
@@ -263,6 +274,25 @@ class Transformer:
         """bf16 working copy <- fp32 master (cast_tree(params, bf16), trainer.py:728); afterwards
         the fused AdamW keeps it current."""
         check(self._L.olmax_cast_f32_to_bf16(stream_ptr(), ptr(self.master), ptr(self.params_bf16), i64(self.num_params)))
+
+    def weight_decay_mask(self, no_decay_modules: Optional[Sequence[str]]):
+        """OptimConfig.build_weight_decay_mask (src/olmax/optim/config.py:94-122) over this model's
+        leaves: a ctypes int32 array in layout order, 0 where the dotted leaf path matches one of the
+        fnmatch patterns (None when nothing is masked).  A pattern that matches nothing warns."""
+        import fnmatch
+        import warnings
+
+        pats = tuple(no_decay_modules or ())
+        if not pats:
+            return None
+        if pats not in self._decay_masks:
+            names = [self.leaf_name(l) for l in self.leaves]
+            for pat in pats:
+                if not any(fnmatch.fnmatch(n, pat) for n in names):
+                    warnings.warn(f"no decay pattern '{pat}' did not match any parameters")
+            mask = [0 if any(fnmatch.fnmatch(n, pat) for pat in pats) else 1 for n in names]
+            self._decay_masks[pats] = (ctypes.c_int32 * len(mask))(*mask)
+        return self._decay_masks[pats]
 
     def named_parameters(self) -> Dict[str, torch.Tensor]:
         return {self.leaf_name(l): self.master[l.offset: l.offset + l.numel].view(l.rows, l.cols) if l.rows > 1
@@ -322,8 +352,9 @@ class Transformer:
         return self.loss
 
     def train_step(self, ids: torch.Tensor, labels: torch.Tensor, *, step: int, lr: float, b1: float = 0.9,
-                   b2: float = 0.999, eps: float = 1e-8, weight_decay: float = 1e-4, decay_embedding: bool = True,
-                   max_grad_norm: Optional[float] = None, overlap_optimizer: bool = True) -> torch.Tensor:
+                   b2: float = 0.999, eps: float = 1e-8, weight_decay: float = 1e-4,
+                   no_decay_modules: Optional[Sequence[str]] = None, max_grad_norm: Optional[float] = None,
+                   overlap_optimizer: bool = True) -> torch.Tensor:
         """loss + gradients + AdamW in one library call (process_microbatch).  With
         ``overlap_optimizer`` each layer's AdamW runs on a second (default-priority) stream while
         the backward pass continues."""
@@ -340,7 +371,7 @@ class Transformer:
             stream_ptr(), opt, ctypes.byref(self.c), self._windows, self._cos, self._sin, ptr(self.master), ptr(self.m),
             ptr(self.v), ptr(self.params_bf16), ptr(ids), ptr(labels), ptr(self.loss), ptr(self.grad_bf16),
             ptr(self.grad_f32), ptr(ws), i64(ws.numel()), i64(step), f32(lr), f32(b1), f32(b2), f32(eps),
-            f32(weight_decay), i32(int(decay_embedding)), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
+            f32(weight_decay), self.weight_decay_mask(no_decay_modules), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
         return self.loss
 
     def accumulate_grads(self, mini_step: int) -> None:
@@ -353,7 +384,7 @@ class Transformer:
                                                   ptr(self.grad_bf16), ptr(self.grad_f32), i32(mini_step)))
 
     def adamw_step_accumulated(self, *, step: int, lr: float, b1: float = 0.9, b2: float = 0.999, eps: float = 1e-8,
-                               weight_decay: float = 1e-4, decay_embedding: bool = True,
+                               weight_decay: float = 1e-4, no_decay_modules: Optional[Sequence[str]] = None,
                                max_grad_norm: Optional[float] = None) -> None:
         """AdamW (and the optional global-norm clip) on the accumulated mean gradient."""
         if self.m is None:
@@ -363,17 +394,18 @@ class Transformer:
         check(self._L.olmax_model_adamw_accumulated(
             stream_ptr(), ctypes.byref(self.c), ptr(self.master), ptr(self.m), ptr(self.v), ptr(self.params_bf16),
             ptr(self.grad_acc), i64(step), f32(lr), f32(b1), f32(b2), f32(eps), f32(weight_decay),
-            i32(int(decay_embedding)), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
+            self.weight_decay_mask(no_decay_modules), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
 
     def init_optimizer_state(self) -> None:
         self.m = torch.zeros(self.num_params, device=self.device, dtype=torch.float32)
         self.v = torch.zeros(self.num_params, device=self.device, dtype=torch.float32)
 
     def adamw_step(self, *, step: int, lr: float, b1: float = 0.9, b2: float = 0.999, eps: float = 1e-8,
-                   weight_decay: float = 1e-4, decay_embedding: bool = True, max_grad_norm: Optional[float] = None):
+                   weight_decay: float = 1e-4, no_decay_modules: Optional[Sequence[str]] = None,
+                   max_grad_norm: Optional[float] = None):
         if self.m is None:
             self.init_optimizer_state()
         check(self._L.olmax_model_adamw(
             stream_ptr(), ctypes.byref(self.c), ptr(self.master), ptr(self.m), ptr(self.v), ptr(self.params_bf16),
             ptr(self.grad_bf16), ptr(self.grad_f32), i64(step), f32(lr), f32(b1), f32(b2), f32(eps), f32(weight_decay),
-            i32(int(decay_embedding)), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
+            self.weight_decay_mask(no_decay_modules), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 30
     missing = [n for n in names if not hasattr(L, n)]
     assert not missing, missing
-    assert L.olmax_abi_version() == 1
+    assert L.olmax_abi_version() == 2
 
 
 def test_layout_queries_on_host():

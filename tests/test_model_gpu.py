@@ -25,18 +25,21 @@ def relerr(a, b):
     return ((a - b).norm() / (b.norm() + 1e-30)).item()
 
 
-def _cfgs(kind, D=128):
+def _cfgs(kind, D=128, full_qk=False):
+    """full_qk: QK-norm over the full projection width instead of per head (attention.py:281-284)."""
     from olmax_amd import TransformerConfig
     gem = kind == "gemma"
     H, K = (4, 2) if gem else (2, 2)
     ocfg = ref.ModelConfig(vocab=512, d_model=256, n_layers=2, n_heads=H, n_kv_heads=K, head_dim=D, hidden=512,
                            layer_type={"default": "pre", "reordered_norm": "reordered", "gemma": "gemma"}[kind],
-                           act="gelu" if gem else "silu", qk_norm=kind != "default", eps=1e-6, rope_theta=1e4,
+                           act="gelu" if gem else "silu", qk_norm=kind != "default" or full_qk, qk_norm_headwise=not full_qk,
+                           eps=1e-6, rope_theta=1e4,
                            rope_theta_layers=[1e4, 1e6] if gem else None, windows=[40, None] if gem else None,
                            attn_softcap=50.0 if gem else 0.0, final_softcap=30.0 if gem else 0.0, tied=gem)
     hcfg = TransformerConfig(vocab_size=512, d_model=256, hidden_size=512, num_layers=2, n_heads=H, n_kv_heads=K,
                              head_dim=D, layer_type=kind, activation="gelu" if gem else "silu",
-                             qk_norm_headwise=kind != "default", norm_eps=1e-6, rope_theta=1e4,
+                             qk_norm_headwise=kind != "default" and not full_qk, qk_norm=kind != "default" or full_qk,
+                             norm_eps=1e-6, rope_theta=1e4,
                              rope_theta_per_layer=[1e4, 1e6] if gem else None,
                              window_size_per_layer=[40, None] if gem else None,
                              attn_logit_softcap=50.0 if gem else 0.0, final_logit_softcap=30.0 if gem else 0.0,
@@ -57,11 +60,11 @@ def _params(ocfg, seed=1):
     return out
 
 
-@pytest.mark.parametrize("kind", ["default", "reordered_norm", "gemma"])
-@pytest.mark.parametrize("D", [128, 64])
-def test_model_loss_and_grads_match_oracle(kind, D):
-    say(f"model grads kind={kind} D={D}")
-    ocfg, hcfg = _cfgs(kind, D)
+@pytest.mark.parametrize("kind,D,full_qk", [(k, D, False) for k in ("default", "reordered_norm", "gemma") for D in (128, 64)]
+                         + [("default", 128, True), ("reordered_norm", 64, True), ("gemma", 128, True)])
+def test_model_loss_and_grads_match_oracle(kind, D, full_qk):
+    say(f"model grads kind={kind} D={D} full-width qk-norm={full_qk}")
+    ocfg, hcfg = _cfgs(kind, D, full_qk)
     B, S = 2, 128
     P = _params(ocfg)
     gen = torch.Generator().manual_seed(5)
@@ -158,12 +161,59 @@ def test_grad_clipping_and_embedding_decay_mask():
     assert not torch.equal(model.named_parameters()["layers.0.mlp.up_proj.weight"], before["layers.0.mlp.up_proj.weight"])
 
 
-@pytest.mark.parametrize("kind", ["reordered_norm", "default", "gemma"])
-def test_single_block_fwd_bwd(kind):
+def test_weight_decay_mask_takes_any_fnmatch_pattern():
+    """no_decay_modules are fnmatch patterns over the leaf paths (src/olmax/optim/config.py:94-122).
+    With all gradients zero AdamW is pure decay: a masked leaf must not move at all, every other
+    leaf becomes p (1 - lr wd); through the whole-model AdamW, the accumulated-gradient AdamW and
+    the overlapped train step (there against the sequential one, with real gradients)."""
+    say("weight-decay mask by pattern")
+    from olmax_amd import AdamWConfig, ConstantSchedule, Trainer
+    import fnmatch
+    ocfg, hcfg = _cfgs("gemma")
+    B, S = 1, 128
+    pats = ["embedding.weight", "*norm.weight", "layers.1.mlp.up_proj.weight"]
+    P = _params(ocfg)
+    for path in ("adamw", "accumulated"):
+        model = hcfg.build(batch_size=B, sequence_length=S)
+        model.load_state_dict(P)
+        before = {k: v.clone() for k, v in model.named_parameters().items()}
+        model.grad_bf16.zero_(); model.grad_f32.zero_()
+        if path == "adamw":
+            model.adamw_step(step=1, lr=0.1, weight_decay=0.25, no_decay_modules=pats)
+        else:
+            model.accumulate_grads(0)
+            model.adamw_step_accumulated(step=1, lr=0.1, weight_decay=0.25, no_decay_modules=pats)
+        n_masked = 0
+        for n, p in model.named_parameters().items():
+            masked = any(fnmatch.fnmatch(n, pat) for pat in pats)
+            n_masked += masked
+            want = before[n] if masked else before[n] * (1 - 0.1 * 0.25)
+            assert (p - want).abs().max().item() <= (0 if masked else 1e-7), (path, n)
+        assert n_masked == 1 + 2 * 6 + 1 + 1  # embedding, six norm weights per gemma layer with QK-norm, final norm, one matrix
+        assert torch.equal(model.params_bf16, model.master.to(BF))  # the bf16 working copy follows the master copy
+    with pytest.warns(UserWarning, match="did not match"):
+        model.weight_decay_mask(["no.such.leaf"])
+    # overlapped (per-layer AdamW on a second stream) == sequential, with the same mask and real gradients
+    hcfg.layer_ac_policy = "nothing_saveable"
+    gen = torch.Generator().manual_seed(4)
+    ids = torch.randint(0, 512, (B * S,), generator=gen, dtype=torch.int32).cuda()
+    outs = []
+    for overlap in (False, True):
+        model = hcfg.build(batch_size=B, sequence_length=S)
+        model.load_state_dict(P)
+        tr = Trainer(model, AdamWConfig(lr=ConstantSchedule(1e-2), weight_decay=0.5, no_decay_modules=pats), overlap_optimizer=overlap)
+        tr.process_microbatch(ids, ids)
+        torch.cuda.synchronize()
+        outs.append(model.master.clone())
+    assert relerr(outs[1], outs[0]) < 1e-5
+
+
+@pytest.mark.parametrize("kind,full_qk", [("reordered_norm", False), ("default", False), ("gemma", False), ("reordered_norm", True)])
+def test_single_block_fwd_bwd(kind, full_qk):
     """BASELINE config 2 at reduced width: one block forward+backward in isolation."""
-    say(f"single block {kind}")
+    say(f"single block {kind} full-width qk-norm={full_qk}")
     from olmax_amd.layer import TransformerBlock
-    ocfg, hcfg = _cfgs(kind)
+    ocfg, hcfg = _cfgs(kind, full_qk=full_qk)
     ocfg.n_layers = hcfg.num_layers = 1
     if kind == "gemma":
         ocfg.windows, ocfg.rope_theta_layers = [40], [1e4]
@@ -364,7 +414,9 @@ def test_fit_loop_logs_every_step_once_with_losses_of_a_manual_run():
 
     tr2 = fresh()
     logged = []
-    tr2.fit(data.DataLoader(3, **kw), max_steps=steps, log_fn=lambda s, m: logged.append((s, m)))
+    dl2 = data.DataLoader(3, **kw)
+    tr2.fit(dl2, max_steps=steps, log_fn=lambda s, m: logged.append((s, m)))
+    assert dl2.get_state()[1] == steps  # the loader is not one batch ahead of what was trained on
     assert tr2.count == steps and [s for s, _ in logged] == list(range(1, steps + 1))
     for (s, m), (loss, lr, gn) in zip(logged, want):
         assert m["optim/lr"] == pytest.approx(lr, rel=1e-6)

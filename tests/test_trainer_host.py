@@ -68,3 +68,56 @@ def test_logging_order_exclusion_and_nan_loss():
     tr.record_metric("train/loss", math.nan)
     with pytest.raises(RuntimeError, match="step 3"):
         tr._log_metrics(None)
+
+
+def test_fit_stops_before_pulling_a_batch_it_will_not_train_on(monkeypatch):
+    """The loop tests completion BEFORE it asks the loader for the next batch (reference
+    src/olmax/train/trainer.py:522-551), so that a loader state saved after fit() points at the first
+    batch that was NOT trained on; a loader that runs dry ends the loop as well."""
+    import torch
+
+    from olmax_amd.optim import AdamWConfig, ConstantSchedule
+
+    class CountingLoader:
+        def __init__(self, n):
+            self.n, self.batches_processed = n, 0
+
+        def __iter__(self):
+            while self.batches_processed < self.n:
+                self.batches_processed += 1  # counted when handed out, as data.DataLoader does
+                yield [(torch.zeros(4, dtype=torch.int32), torch.zeros(4, dtype=torch.int32))]
+
+        def get_state(self):
+            return (0, self.batches_processed, 0)
+
+    monkeypatch.setattr(torch.cuda, "synchronize", lambda *a, **k: None)
+    tr = Trainer.__new__(Trainer)  # host logic only: the step itself is replaced
+    tr.count, tr.optim = 0, AdamWConfig(lr=ConstantSchedule(1e-3))
+
+    def fake_train_batch(batch):
+        tr.count += 1
+        return 1.0 / tr.count
+
+    tr.train_batch = fake_train_batch
+    dl = CountingLoader(10)
+    logged = []
+    tr.fit(dl, max_steps=4, log_fn=lambda s, m: logged.append(s))
+    assert tr.count == 4 and dl.get_state()[1] == 4 and logged == [1, 2, 3, 4]
+    tr.fit(dl, max_steps=4)   # already complete: nothing is pulled
+    assert dl.get_state()[1] == 4
+    tr.fit(dl, max_steps=100)  # the loader runs dry after 6 more
+    assert tr.count == 10 and dl.get_state()[1] == 10
+
+
+def test_adamw_config_decay_patterns():
+    """fnmatch patterns over dotted leaf paths (src/olmax/optim/config.py:94-122; the reference's own
+    mask test, src/test/optim/config_test.py:36-47, on its names)."""
+    from olmax_amd.optim import AdamWConfig
+
+    c = AdamWConfig(no_decay_modules=["gate_proj.bias", "down_proj.bias", "up_proj.bias"])
+    for m in ("gate_proj", "down_proj", "up_proj"):
+        assert c.decays(f"{m}.weight") is True and c.decays(f"{m}.bias") is False
+    c = AdamWConfig(no_decay_modules=["embedding.weight", "*norm.weight"])
+    assert not c.decays("embedding.weight") and not c.decays("layers.3.attention.q_norm.weight") and not c.decays("norm.weight")
+    assert c.decays("layers.3.mlp.up_proj.weight") and c.decays("lm_head.proj.weight")
+    assert AdamWConfig().decays("embedding.weight")
