@@ -13,7 +13,18 @@
  *    dimension is contiguous.  bf16 storage, fp32 accumulation and statistics.
  *  - Return 0 on success; negative on an argument error detected on the host before any
  *    launch (olmax_last_error_string() gives the thread-local message).  Nothing throws.
- *  - Calls hold no mutable global state; except where noted they never allocate.
+ *  - Compute entry points never allocate device memory and may be called from any host thread;
+ *    what they keep between calls is immutable once set (kernel attributes, set once under
+ *    std::call_once; the device's CU count) or per thread (the last error string, one HIP event of
+ *    olmax_model_train_step).  The exceptions are the three process-wide DIAGNOSTIC switches at
+ *    the end of this file (tile override, GEMM event profile, profiler ranges) and
+ *    olmax_attn_bwd_noalloc, whose scratch array is shared by all calls on a GPU.
+ *  - Arguments are flat lists of pointers, sizes and scalars (no parameter structs except the
+ *    whole-model configuration); an op that needs scratch takes `workspace` + `workspace_bytes`
+ *    and has a pure `<op>_workspace_bytes` companion.
+ *  - Token ids follow NumPy/JAX indexing of `weight[ids]`: a negative id counts from the end and
+ *    what is still outside [0, vocab) is clamped (gather and its scatter-add transpose alike);
+ *    labels outside [0, vocab) follow the reference's one-hot semantics (see olmax_cross_entropy).
  */
 #ifndef OLMAX_HIP_H
 #define OLMAX_HIP_H
@@ -45,17 +56,6 @@ int32_t olmax_abi_version(void);
 int32_t olmax_gemm_bf16(olmax_stream_t stream, const void* A, const void* B, void* C, const void* R,
                         int32_t M, int32_t N, int32_t K, int64_t lda, int64_t ldb, int64_t ldc,
                         int64_t ldr, int32_t a_layout, int32_t b_layout, int32_t out_f32);
-/* Test/tuning hook: force the MFMA tile variant (0 = automatic). */
-void olmax_gemm_set_tile(int tile);
-/* Diagnostic: record a HIP-event pair on the launch stream around every MFMA GEMM launch
- * between begin and end (allocates events; not for graph capture).  end() waits for them and
- * aggregates per kernel instantiation: key = tile | a_kc<<12 | b_kc<<13 | has_res<<14 |
- * out_f32<<15 | glu_epilogue<<16; ms = summed durations, flops / bytes = summed algorithmic
- * work (2MNK; operands and result moved once).  Returns the number of distinct keys written
- * (at most cap). */
-void olmax_gemm_profile_begin(void);
-int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, double* bytes, int64_t* launches,
-                               int32_t cap);
 
 /* ---- RMSNorm: rms_norm, src/olmax/nn/functional.py:51-67; RMSNorm.forward,
  * src/olmax/nn/normalization.py:85-87.  w may be NULL (no scale). */
@@ -173,13 +173,6 @@ int32_t olmax_lmhead_ce(olmax_stream_t stream, const void* h, const void* W, con
                         float* loss, void* dh, void* dW, void* workspace, int64_t workspace_bytes,
                         int64_t T, int32_t d, int32_t V, int32_t ignore_index, float softcap,
                         int32_t dw_f32);
-
-/* ---- Profiler ranges: the counterpart of the reference's jax.named_scope annotations and
- * ProfilerCallback (src/olmax/train/callbacks/profiler.py:33-50).  on != 0: the whole-model entry
- * points emit roctx ranges ("olmax.layers.<l>.forward" / ".backward", "olmax.lm_head_and_loss")
- * on the calling host thread, visible to rocprofv3 --marker-trace.  Needs libroctx64.so at run
- * time; returns an error (and stays off) without it. */
-int32_t olmax_set_profiler_ranges(int32_t on);
 
 /* ---- Synthetic token batches: _randomize_start_offsets, src/olmax/data/utils.py:12-33:
  * inputs[b, s] = (s + start_offsets[b]) mod V, targets = inputs + 1 (so a target equals V when
@@ -340,6 +333,29 @@ int32_t olmax_block_bwd(olmax_stream_t stream, const olmax_model_config* cfg, co
                         const olmax_block_grads* g, int32_t window, const float* cos_t,
                         const float* sin_t, const void* x, const void* dy, void* dx, void* acts,
                         int64_t acts_bytes, void* tmp, int64_t tmp_bytes);
+
+/* =====================================================================================
+ * Diagnostics.  Process-wide switches (atomics): they change what EVERY thread's later calls do,
+ * are meant for tests, tuning and profiling runs, and are not for use while other threads are
+ * inside the library or under graph capture.
+ * ===================================================================================== */
+/* Force the MFMA tile variant of olmax_gemm_bf16 (0 = automatic, 128, 256).  While set, the
+ * fused GLU / RoPE projections take their unfused paths (same results). */
+void olmax_gemm_set_tile(int tile);
+/* Record a HIP-event pair on the launch stream around every MFMA GEMM launch between begin and
+ * end (allocates events).  end() waits for them and aggregates per kernel instantiation:
+ * key = tile | a_kc<<12 | b_kc<<13 | has_res<<14 | out_f32<<15 | glu_epilogue<<16 |
+ * rope_epilogue<<17; ms = summed durations, flops / bytes = summed algorithmic work (2MNK;
+ * operands and result moved once).  Returns the number of distinct keys written (at most cap). */
+void olmax_gemm_profile_begin(void);
+int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, double* bytes, int64_t* launches,
+                               int32_t cap);
+/* Profiler ranges: the counterpart of the reference's jax.named_scope annotations and
+ * ProfilerCallback (src/olmax/train/callbacks/profiler.py:33-50).  on != 0: the whole-model entry
+ * points emit roctx ranges ("olmax.layers.<l>.forward" / ".backward", "olmax.lm_head_and_loss")
+ * on the calling host thread, visible to rocprofv3 --marker-trace.  Needs a roctx library at run
+ * time; returns an error (and stays off) without it. */
+int32_t olmax_set_profiler_ranges(int32_t on);
 
 #ifdef __cplusplus
 }

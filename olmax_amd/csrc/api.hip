@@ -2,6 +2,8 @@
 #include "common.h"
 #include <string.h>
 #include <dlfcn.h>
+#include <atomic>
+#include <mutex>
 
 static thread_local char g_err[512] = "";
 
@@ -24,9 +26,11 @@ extern "C" int32_t olmax_abi_version(void) { return 2; }
 // time the first time ranges are switched on; without it the switch reports an error and stays off.
 static int (*g_roctx_push)(const char*) = nullptr;
 static int (*g_roctx_pop)(void) = nullptr;
-static bool g_ranges_on = false;
+static std::atomic<bool> g_ranges_on{false};  // diagnostic switch, process-wide
+static std::mutex g_roctx_mu;
 
 extern "C" int32_t olmax_set_profiler_ranges(int32_t on) {
+  std::lock_guard<std::mutex> lock(g_roctx_mu);
   if (on && !g_roctx_push) {
     // rocprofv3 listens to the SDK's roctx library; the roctracer one serves the older tools
     const char* names[] = {"librocprofiler-sdk-roctx.so", "librocprofiler-sdk-roctx.so.1", "libroctx64.so", "libroctx64.so.4"};

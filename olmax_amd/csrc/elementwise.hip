@@ -152,7 +152,14 @@ __global__ __launch_bounds__(256) void sequential_tokens_kernel(const int32_t* _
 }
 
 // ------------------------------------------------------------------ embedding
-// ids outside [0, V) are clamped (memory safety; the data path never produces them).
+// ids follow NumPy/JAX indexing of `weight[ids]` (src/olmax/nn/embedding.py:32): a negative id
+// counts from the end, and what is still outside [0, V) is clamped (JAX's gather mode for
+// out-of-bounds reads; upstream semantics, the data path never produces such ids).  The
+// scatter-add is the transpose of exactly that gather.
+__device__ __forceinline__ int wrap_clamp_id(int id, int V) {
+  if (id < 0) id += V;
+  return id < 0 ? 0 : (id >= V ? V - 1 : id);
+}
 __global__ __launch_bounds__(256) void embed_fwd_kernel(const int32_t* __restrict__ ids,
                                                         const bf16* __restrict__ W,
                                                         bf16* __restrict__ out, int64_t T, int d,
@@ -162,16 +169,14 @@ __global__ __launch_bounds__(256) void embed_fwd_kernel(const int32_t* __restric
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t t = i / cpr;
     const int c = (int)(i % cpr) * 8;
-    int id = ids[t];
-    id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+    const int id = wrap_clamp_id(ids[t], V);
     *reinterpret_cast<u32x4*>(out + t * d + c) = *reinterpret_cast<const u32x4*>(W + (int64_t)id * d + c);
   }
 }
 __global__ void embed_fwd_scalar(const int32_t* ids, const bf16* W, bf16* out, int64_t T, int d, int V) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= T * d) return;
-  int id = ids[i / d];
-  id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+  const int id = wrap_clamp_id(ids[i / d], V);
   out[i] = W[(int64_t)id * d + i % d];
 }
 // dW[ids[t], :] += dh[t, :]   (fp32 accumulate; duplicates sum through atomics)
@@ -182,8 +187,7 @@ __global__ __launch_bounds__(256) void embed_bwd_kernel(const int32_t* __restric
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < T * d; i += (int64_t)gridDim.x * 256) {
     const int64_t t = i / d;
     const int c = (int)(i % d);
-    int id = ids[t];
-    if (id < 0 || id >= V) continue;
+    const int id = wrap_clamp_id(ids[t], V);
     atomicAdd(&dW[(int64_t)id * d + c], bf2f(dh[i]));
   }
 }

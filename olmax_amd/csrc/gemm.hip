@@ -32,6 +32,7 @@
 // every XCD one contiguous run of tiles; runs walk the tile grid in column groups so that
 // the A row-panels and B column-panels a single L2 sees are re-used.
 #include "common.h"
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 #include <vector>
@@ -52,7 +53,7 @@ struct ProfRec {
   double bytes;  // algorithmic: every operand and the result moved once
   int key;  // tile | a_kc<<12 | b_kc<<13 | has_res<<14 | out_f32<<15
 };
-bool g_prof_on = false;
+std::atomic<bool> g_prof_on{false};  // diagnostic switch, process-wide
 std::vector<ProfRec> g_prof;
 std::mutex g_prof_mu;
 
@@ -591,11 +592,8 @@ int launch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   constexpr int SMEM = 2 * (BM + BN) * BK * 2;
   auto kern = gemm_bf16_kernel<BM, BN, WM, WN, A_KC, B_KC, HAS_RES, OUT_F32>;
-  static bool attr_set = false;  // one-time, idempotent
-  if (!attr_set) {
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-    attr_set = true;
-  }
+  static std::once_flag attr_once;  // per instantiation
+  std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM); });
   const int tm = M / BM, tn = N / BN;
   ProfRec rec{};
   if (g_prof_on) {
@@ -624,11 +622,8 @@ int launch_glu(hipStream_t s, const bf16* A, const bf16* B, bf16* gu, bf16* act,
                int64_t ldb, int64_t ldgu, int64_t ldact) {
   constexpr int SMEM = 2 * (256 + 256) * BK * 2;
   auto kern = gemm_bf16_kernel<256, 256, 128, 64, true, true, false, false, GLU>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-    attr_set = true;
-  }
+  static std::once_flag attr_once;  // per instantiation
+  std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM); });
   const int tm = M / 256, tn = F / 128;
   ProfRec rec{};
   if (g_prof_on) {
@@ -663,7 +658,7 @@ int dispatch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf
                                                                      ldb, ldc, ldr);
 }
 
-int g_force_tile = 0;
+std::atomic<int> g_force_tile{0};  // diagnostic override, process-wide
 
 }  // namespace
 
@@ -731,19 +726,20 @@ extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void
   const bf16* r = (const bf16*)R;
   const bool vec_ok = aligned16(A) && aligned16(B) && (lda % 8 == 0) && (ldb % 8 == 0);
   int tile = 0;
+  const int force_tile = g_force_tile.load(std::memory_order_relaxed);
   if (vec_ok && K % BK == 0) {
     if (M % 256 == 0 && N % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 128) tile = 256;
     else if (M % 128 == 0 && N % 128 == 0) tile = 128;
   }
-  if (g_force_tile && tile) {
-    if (g_force_tile == 256 && M % 256 == 0 && N % 256 == 0) tile = 256;
-    if (g_force_tile == 128) tile = 128;
+  if (force_tile && tile) {
+    if (force_tile == 256 && M % 256 == 0 && N % 256 == 0) tile = 256;
+    if (force_tile == 128) tile = 128;
   }
   // Wave quantisation: with one 256x256 tile per CU per round, a last round that fills less
   // than half of the CUs (e.g. 1376 tiles = 5.375 rounds on 256 CUs) costs a whole round.
   // Such a problem is cut along M or N into a part whose tile count is a whole number of
   // rounds and a remainder that goes through this function again (and gets smaller tiles).
-  if (tile == 256 && !g_force_tile) {
+  if (tile == 256 && !force_tile) {
     const int ncu = device_cu_count();
     const int tm = M / 256, tn = N / 256;
     const int64_t tiles = (int64_t)tm * tn;
@@ -817,15 +813,12 @@ extern "C" int32_t olmax_gemm_rope_bf16(hipStream_t stream, const void* X, const
   OLMAX_CHECK(ldx >= K && ldw >= K && ldo >= N, OLMAX_ERR_SHAPE, "olmax_gemm_rope_bf16: leading dimension smaller than row length");
   const bool fits = aligned16(X) && aligned16(W) && aligned16(out) && aligned16(cos_t) && aligned16(sin_t) && ldx % 8 == 0 &&
                     ldw % 8 == 0 && ldo % 8 == 0 && K % BK == 0 && M % 256 == 0 && N % 256 == 0 && rope_heads % 2 == 0 &&
-                    (int64_t)(M / 256) * (N / 256) >= 128 && !g_force_tile;
+                    (int64_t)(M / 256) * (N / 256) >= 128 && !g_force_tile.load(std::memory_order_relaxed);
   if (fits) {
     constexpr int SMEM = 2 * (256 + 256) * BK * 2;
     auto kern = gemm_bf16_kernel<256, 256, 128, 64, true, true, false, false, 3>;
-    static bool attr_set = false;
-    if (!attr_set) {
-      (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-      attr_set = true;
-    }
+    static std::once_flag attr_once;  // per instantiation
+    std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM); });
     const int tm = M / 256, tn = N / 256;
     ProfRec rec{};
     if (g_prof_on) {
@@ -867,7 +860,7 @@ extern "C" int32_t olmax_gemm_glu_bf16(hipStream_t stream, const void* X, const 
   OLMAX_CHECK(ldx >= K && ldw >= K && ldact >= F && (!gu_out || ldgu >= 2 * (int64_t)F), OLMAX_ERR_SHAPE,
               "olmax_gemm_glu_bf16: leading dimension smaller than row length");
   const bool fits = aligned16(X) && aligned16(W) && ldx % 8 == 0 && ldw % 8 == 0 && K % BK == 0 && M % 256 == 0 &&
-                    F % 128 == 0 && (int64_t)(M / 256) * (F / 128) >= 128 && !g_force_tile;
+                    F % 128 == 0 && (int64_t)(M / 256) * (F / 128) >= 128 && !g_force_tile.load(std::memory_order_relaxed);
   if (fits) {
     if (act == 0) return launch_glu<1>(stream, (const bf16*)X, (const bf16*)W, (bf16*)gu_out, (bf16*)act_out, M, F, K, ldx, ldw, ldgu, ldact);
     return launch_glu<2>(stream, (const bf16*)X, (const bf16*)W, (bf16*)gu_out, (bf16*)act_out, M, F, K, ldx, ldw, ldgu, ldact);

@@ -427,6 +427,13 @@ def test_embedding():
     dW = ops.embed_bwd(ids.cuda(), dh.cuda(), V)
     want = ref.embed_bwd(ids, dh.double(), V)
     assert (dW.cpu().double() - want).abs().max() < 1e-5
+    # ids outside [0, V): NumPy/JAX indexing (negative counts from the end, the rest is clamped),
+    # and the scatter-add is the transpose of that gather
+    odd = torch.tensor([-1, V, V + 5, -V - 3, 2], dtype=torch.int32)
+    rows = torch.tensor([V - 1, V - 1, V - 1, 0, 2])
+    assert torch.equal(ops.embed_fwd(odd.cuda(), W.cuda()).cpu(), W[rows])
+    dh5 = bfr(5, d, seed=4)
+    assert (ops.embed_bwd(odd.cuda(), dh5.cuda(), V).cpu().double() - ref.embed_bwd(rows, dh5.double(), V)).abs().max() < 1e-5
     # odd width goes through the scalar path
     W2 = bfr(V, 13, seed=3)
     assert torch.equal(ops.embed_fwd(ids.cuda(), W2.cuda()).cpu(), W2[ids.long()])
