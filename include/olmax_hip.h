@@ -200,6 +200,13 @@ int32_t olmax_adamw_dscale(olmax_stream_t stream, float* p, const void* g, float
                            void* shadow_bf16, int64_t n, int32_t grad_is_bf16, float lr, float b1,
                            float b2, float eps, float wd, int64_t step, float grad_scale,
                            const float* grad_scale_dev);
+/* As olmax_adamw_dscale with the step-dependent scalars in device memory: hyper_dev = fp32
+ * {lr, 1 - b1^step, 1 - b2^step}, written by earlier work on the same stream.  For hosts whose
+ * schedule and step count are device values (optax's inject_hyperparams state inside a jitted
+ * step, src/olmax/optim/config.py:141-148): no host read-back, no recompilation per step. */
+int32_t olmax_adamw_dev(olmax_stream_t stream, float* p, const void* g, float* m, float* v, void* shadow_bf16,
+                        int64_t n, int32_t grad_is_bf16, float b1, float b2, float eps, float wd,
+                        const float* hyper_dev, const float* grad_scale_dev);
 /* *out += sum(g^2): building block of get_global_norm, src/olmax/jax_utils.py:88-102. */
 int32_t olmax_sumsq(olmax_stream_t stream, const void* g, int64_t n, int32_t is_bf16, float* out);
 
@@ -278,11 +285,13 @@ int32_t olmax_model_loss(olmax_stream_t stream, const olmax_model_config* cfg, c
  * (src/olmax/optim/config.py:94-122; the benchmark exempts "embedding.weight",
  * src/integration_tests/train_transformer.py:388); NULL = every leaf decays.  max_grad_norm > 0 applies
  * clip_grads_by_global_norm (src/olmax/optim/utils.py:22-38); norm_scratch: device float[2], left holding
- * {clip factor, gradient norm}. */
+ * {clip factor, gradient norm}.  hyper_dev (optional, as in olmax_adamw_dev): device fp32
+ * {lr, 1 - b1^step, 1 - b2^step}; when given, the host `step` and `lr` arguments are ignored. */
 int32_t olmax_model_adamw(olmax_stream_t stream, const olmax_model_config* cfg, float* master,
                           float* m, float* v, void* params_bf16, const void* grad_bf16,
                           const float* grad_f32, int64_t step, float lr, float b1, float b2, float eps,
-                          float wd, const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch);
+                          float wd, const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch,
+                          const float* hyper_dev);
 
 /* Gradient accumulation over micro-batches: optax.MultiSteps as built at
  * src/olmax/optim/config.py:153-154 and driven once per micro-batch by train_batch,
@@ -298,7 +307,8 @@ int32_t olmax_model_grad_accumulate(olmax_stream_t stream, const olmax_model_con
 int32_t olmax_model_adamw_accumulated(olmax_stream_t stream, const olmax_model_config* cfg, float* master,
                                       float* m, float* v, void* params_bf16, const float* acc, int64_t step,
                                       float lr, float b1, float b2, float eps, float wd,
-                                      const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch);
+                                      const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch,
+                                      const float* hyper_dev);
 
 /* process_microbatch, src/olmax/train/trainer.py:759-777: loss + gradients + AdamW in one call.
  * opt_stream (optional, default priority, != stream): when given, clipping is off and the config
@@ -311,7 +321,8 @@ int32_t olmax_model_train_step(olmax_stream_t stream, olmax_stream_t opt_stream,
                                void* params_bf16, const int32_t* ids, const int32_t* labels, float* loss,
                                void* grad_bf16, float* grad_f32, void* workspace, int64_t workspace_bytes,
                                int64_t step, float lr, float b1, float b2, float eps, float wd,
-                               const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch);
+                               const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch,
+                               const float* hyper_dev);
 
 /* Single transformer block in isolation (any of the three orderings). */
 typedef struct {

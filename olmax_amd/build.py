@@ -57,6 +57,43 @@ def build_all(force: bool = True, jobs: int = 8) -> Path:
     return LIB
 
 
+FFI_SRC = HERE / "ffi" / "olmax_ffi.cc"
+FFI_LIB = HERE / "libolmax_ffi.so"
+
+
+def xla_ffi_include_dir():
+    """Directory that holds xla/ffi/api/ffi.h (it ships inside jaxlib), or None.  $OLMAX_XLA_FFI_INCLUDE
+    overrides the lookup through jax.ffi.include_dir()."""
+    cand = os.environ.get("OLMAX_XLA_FFI_INCLUDE")
+    if not cand:
+        try:
+            import jax.ffi  # noqa: WPS433 - optional dependency, absent in this image
+
+            cand = jax.ffi.include_dir()
+        except Exception:
+            return None
+    return cand if cand and (Path(cand) / "xla" / "ffi" / "api" / "ffi.h").exists() else None
+
+
+def build_ffi_adapter():
+    """Compile the XLA-FFI adapter (ffi/olmax_ffi.cc -> libolmax_ffi.so, linked against
+    libolmax_hip.so) when the XLA FFI headers are installed; returns the library path, or None
+    (with a note on stderr) when they are not.  Nothing stands in for missing headers."""
+    inc = xla_ffi_include_dir()
+    if inc is None:
+        print("olmax_amd.build: XLA FFI headers (xla/ffi/api/ffi.h, shipped with jaxlib) not found: "
+              "libolmax_ffi.so not built", file=sys.stderr)
+        return None
+    cmd = [HIPCC, "-x", "c++", "-D__HIP_PLATFORM_AMD__", "-O2", "-std=c++17", "-fPIC", "-shared", "-I", inc,
+           "-I", str(HERE.parent / "include"), "-I", "/opt/rocm/include", str(FFI_SRC), "-o", str(FFI_LIB),
+           "-L", str(HERE), "-lolmax_hip", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {FFI_SRC.name}:\n{r.stderr[-4000:]}")
+    return FFI_LIB
+
+
 if __name__ == "__main__":
     p = build_all(force="--force" in sys.argv)
     print(p)
+    build_ffi_adapter()

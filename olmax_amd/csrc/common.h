@@ -147,4 +147,4 @@ __device__ __forceinline__ float act_gelu(float g) {
 // elementwise.hip, library-internal: olmax_adamw_dscale with the grid size (workgroups) exposed.
 int olmax_adamw_grid(hipStream_t stream, float* p, const void* g, float* m, float* v, void* shadow_bf16, int64_t n,
                      int32_t grad_is_bf16, float lr, float b1, float b2, float eps, float wd, int64_t step,
-                     float grad_scale, const float* grad_scale_dev, int grid_cap);
+                     float grad_scale, const float* grad_scale_dev, int grid_cap, const float* hyper_dev = nullptr);

@@ -194,13 +194,20 @@ __global__ __launch_bounds__(256) void embed_bwd_kernel(const int32_t* __restric
 
 // ------------------------------------------------------------------ AdamW
 // p, m, v fp32 in place; g bf16 or fp32; optional bf16 working copy of the new p.
-// bc1 = 1 - b1^t, bc2 = 1 - b2^t (computed on the host in double).
+// bc1 = 1 - b1^t, bc2 = 1 - b2^t (computed on the host in double), or, with hyper_dev, lr and the
+// two bias corrections read from device memory (a host whose schedule and step count live on
+// the device, like optax's injected hyper-parameters inside a jitted step).
 template <bool G_BF16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(16))) void adamw_kernel(
     float* __restrict__ p, const void* __restrict__ gv, float* __restrict__ m, float* __restrict__ v,
     bf16* __restrict__ shadow, int64_t n, float lr, float b1, float b2, float eps, float wd, float bc1,
-    float bc2, float gscale, const float* __restrict__ gscale_dev) {
+    float bc2, float gscale, const float* __restrict__ gscale_dev, const float* __restrict__ hyper_dev) {
   if (gscale_dev) gscale *= *gscale_dev;
+  if (hyper_dev) {  // step-dependent scalars from device memory (wave-uniform scalar loads)
+    lr = hyper_dev[0];
+    bc1 = hyper_dev[1];
+    bc2 = hyper_dev[2];
+  }
   const int64_t n4 = n / 4;
   const float ibc1 = 1.f / bc1, ibc2 = 1.f / bc2, omb1 = 1.f - b1, omb2 = 1.f - b2;
   // Every element is touched exactly once: streaming (non-temporal) accesses keep the 28 B/param
@@ -406,14 +413,24 @@ extern "C" int32_t olmax_adamw_dscale(hipStream_t stream, float* p, const void* 
                                       const float* grad_scale_dev) {
   // two workgroups per CU: the fastest grid when the kernel has the GPU to itself
   return olmax_adamw_grid(stream, p, g, m, v, shadow_bf16, n, grad_is_bf16, lr, b1, b2, eps, wd, step, grad_scale,
-                          grad_scale_dev, 512);
+                          grad_scale_dev, 512, nullptr);
+}
+
+// As olmax_adamw_dscale with lr and the bias corrections in device memory:
+// hyper_dev = {lr, 1 - b1^step, 1 - b2^step} (fp32), written by earlier work on the same stream.
+extern "C" int32_t olmax_adamw_dev(hipStream_t stream, float* p, const void* g, float* m, float* v, void* shadow_bf16,
+                                   int64_t n, int32_t grad_is_bf16, float b1, float b2, float eps, float wd,
+                                   const float* hyper_dev, const float* grad_scale_dev) {
+  OLMAX_CHECK(hyper_dev, OLMAX_ERR_ARG, "olmax_adamw_dev: hyper_dev is null");
+  return olmax_adamw_grid(stream, p, g, m, v, shadow_bf16, n, grad_is_bf16, 0.f, b1, b2, eps, wd, 1, 1.f, grad_scale_dev, 512,
+                          hyper_dev);
 }
 
 // Library-internal form with the grid size exposed: the overlapped train step runs it with one
 // workgroup per CU on its second stream, which disturbs the GEMMs it shares the GPU with least.
 int olmax_adamw_grid(hipStream_t stream, float* p, const void* g, float* m, float* v, void* shadow_bf16, int64_t n,
                      int32_t grad_is_bf16, float lr, float b1, float b2, float eps, float wd, int64_t step,
-                     float grad_scale, const float* grad_scale_dev, int grid_cap) {
+                     float grad_scale, const float* grad_scale_dev, int grid_cap, const float* hyper_dev) {
   if (n == 0) return OLMAX_OK;
   OLMAX_CHECK(p && g && m && v, OLMAX_ERR_ARG, "olmax_adamw: null pointer");
   OLMAX_CHECK(n >= 0 && step >= 1, OLMAX_ERR_ARG, "olmax_adamw: n must be >= 0 and step >= 1 (1-based)");
@@ -424,9 +441,9 @@ int olmax_adamw_grid(hipStream_t stream, float* p, const void* g, float* m, floa
   const float bc2 = (float)(1.0 - pow((double)b2, (double)step));
   const int grid = grid_1d((n + 3) / 4, grid_cap);
   if (grad_is_bf16)
-    hipLaunchKernelGGL(adamw_kernel<true>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale, grad_scale_dev);
+    hipLaunchKernelGGL(adamw_kernel<true>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale, grad_scale_dev, hyper_dev);
   else
-    hipLaunchKernelGGL(adamw_kernel<false>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale, grad_scale_dev);
+    hipLaunchKernelGGL(adamw_kernel<false>, dim3(grid), dim3(256), 0, stream, p, g, m, v, (bf16*)shadow_bf16, n, lr, b1, b2, eps, wd, bc1, bc2, grad_scale, grad_scale_dev, hyper_dev);
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
 }

@@ -511,7 +511,8 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
 // NULL: every leaf decays) is the weight-decay mask of AdamWConfig.build.
 int adamw_leaves(hipStream_t s, const olmax_leaf* leaves, int begin, int end, float* master, float* mom, float* var,
                  bf16* shadow, const bf16* G, const float* grad_f32, int64_t step, float lr, float b1, float b2,
-                 float eps, float wd, const int32_t* leaf_decay, const float* dscale, int grid_cap = 512) {
+                 float eps, float wd, const int32_t* leaf_decay, const float* dscale, int grid_cap = 512,
+                 const float* hyper_dev = nullptr) {
   auto decays = [&](int i) { return !leaf_decay || leaf_decay[i] != 0; };
   int i = begin;
   while (i < end) {
@@ -519,7 +520,7 @@ int adamw_leaves(hipStream_t s, const olmax_leaf* leaves, int begin, int end, fl
     const float lwd = decays(i) ? wd : 0.f;
     if (lf.grad_f32) {
       RC(olmax_adamw_grid(s, master + lf.offset, grad_f32 + lf.grad_f32_offset, mom + lf.offset, var + lf.offset,
-                          shadow + lf.offset, lf.numel, 0, lr, b1, b2, eps, lwd, step, 1.f, dscale, grid_cap));
+                          shadow + lf.offset, lf.numel, 0, lr, b1, b2, eps, lwd, step, 1.f, dscale, grid_cap, hyper_dev));
       i++;
     } else {
       int64_t n = lf.numel;
@@ -529,7 +530,7 @@ int adamw_leaves(hipStream_t s, const olmax_leaf* leaves, int begin, int end, fl
         j++;
       }
       RC(olmax_adamw_grid(s, master + lf.offset, G + lf.offset, mom + lf.offset, var + lf.offset, shadow + lf.offset, n, 1,
-                          lr, b1, b2, eps, lwd, step, 1.f, dscale, grid_cap));
+                          lr, b1, b2, eps, lwd, step, 1.f, dscale, grid_cap, hyper_dev));
       i = j;
     }
   }
@@ -550,6 +551,7 @@ struct OverlapCtx {
   int64_t step;
   float lr, b1, b2, eps, wd;
   const int32_t* leaf_decay;
+  const float* hyper_dev;
   // 0: launch as soon as the gradients are final; else at that StepHook point.  Measured on
   // the 7B step: AdamW as a one-workgroup-per-CU grid of 32-register waves launched at once
   // (it then shares CUs with the next block's forward GEMMs, whose waves leave it 32 registers
@@ -590,7 +592,7 @@ int overlap_launch(OverlapCtx* x, int layer) {
   if (hipEventRecord(x->ev, x->main) != hipSuccess || hipStreamWaitEvent(x->opt, x->ev, 0) != hipSuccess)
     return olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_model_train_step: event record/wait failed");
   return adamw_leaves(x->opt, x->leaves, begin, end, x->master, x->mom, x->var, x->shadow, x->G, x->grad_f32, x->step, x->lr,
-                      x->b1, x->b2, x->eps, x->wd, x->leaf_decay, nullptr, 256);
+                      x->b1, x->b2, x->eps, x->wd, x->leaf_decay, nullptr, 256, x->hyper_dev);
 }
 
 __global__ void clip_scale_kernel(const float* sumsq, float max_norm, float* out) {
@@ -717,10 +719,11 @@ extern "C" int32_t olmax_model_loss(hipStream_t s, const olmax_model_config* c, 
 extern "C" int32_t olmax_model_adamw(hipStream_t s, const olmax_model_config* c, float* master, float* mom, float* var,
                                      void* params_bf16, const void* grad_bf16, const float* grad_f32, int64_t step,
                                      float lr, float b1, float b2, float eps, float wd, const int32_t* leaf_decay,
-                                     float max_grad_norm, float* norm_scratch) {
+                                     float max_grad_norm, float* norm_scratch, const float* hyper_dev) {
   RC(check_cfg(c));
   OLMAX_CHECK(master && mom && var && params_bf16 && grad_bf16 && grad_f32, OLMAX_ERR_ARG, "olmax_model_adamw: null pointer");
-  OLMAX_CHECK(step >= 1, OLMAX_ERR_ARG, "olmax_model_adamw: step is 1-based");
+  OLMAX_CHECK(step >= 1 || hyper_dev, OLMAX_ERR_ARG, "olmax_model_adamw: step is 1-based");
+  if (hyper_dev) step = 1;  // unused by the kernels then
   OLMAX_CHECK(max_grad_norm <= 0.f || norm_scratch, OLMAX_ERR_ARG, "olmax_model_adamw: clipping needs norm_scratch");
   const int nleaf = olmax_model_layout(c, nullptr, 0);
   olmax_leaf* leaves = new olmax_leaf[nleaf];
@@ -742,7 +745,7 @@ extern "C" int32_t olmax_model_adamw(hipStream_t s, const olmax_model_config* c,
       dscale = norm_scratch;
     }
   }
-  if (!rc) rc = adamw_leaves(s, leaves, 0, nleaf, master, mom, var, shadow, G, grad_f32, step, lr, b1, b2, eps, wd, leaf_decay, dscale);
+  if (!rc) rc = adamw_leaves(s, leaves, 0, nleaf, master, mom, var, shadow, G, grad_f32, step, lr, b1, b2, eps, wd, leaf_decay, dscale, 512, hyper_dev);
   delete[] leaves;
   return rc;
 }
@@ -783,10 +786,11 @@ extern "C" int32_t olmax_model_grad_accumulate(hipStream_t s, const olmax_model_
 extern "C" int32_t olmax_model_adamw_accumulated(hipStream_t s, const olmax_model_config* c, float* master, float* mom,
                                                  float* var, void* params_bf16, const float* acc, int64_t step, float lr,
                                                  float b1, float b2, float eps, float wd, const int32_t* leaf_decay,
-                                                 float max_grad_norm, float* norm_scratch) {
+                                                 float max_grad_norm, float* norm_scratch, const float* hyper_dev) {
   RC(check_cfg(c));
   OLMAX_CHECK(master && mom && var && params_bf16 && acc, OLMAX_ERR_ARG, "olmax_model_adamw_accumulated: null pointer");
-  OLMAX_CHECK(step >= 1, OLMAX_ERR_ARG, "olmax_model_adamw_accumulated: step is 1-based");
+  OLMAX_CHECK(step >= 1 || hyper_dev, OLMAX_ERR_ARG, "olmax_model_adamw_accumulated: step is 1-based");
+  if (hyper_dev) step = 1;
   OLMAX_CHECK(max_grad_norm <= 0.f || norm_scratch, OLMAX_ERR_ARG, "olmax_model_adamw_accumulated: clipping needs norm_scratch");
   const Layout L = layout_of(c);
   bf16* shadow = (bf16*)params_bf16;
@@ -808,8 +812,8 @@ extern "C" int32_t olmax_model_adamw_accumulated(hipStream_t s, const olmax_mode
     int64_t n = leaves[i].numel;
     while (j < nleaf && decays(j) == decays(i) && leaves[j].offset == leaves[i].offset + n) n += leaves[j++].numel;
     const int64_t o = leaves[i].offset;
-    rc = olmax_adamw_dscale(s, master + o, acc + o, mom + o, var + o, shadow + o, n, 0, lr, b1, b2, eps, decays(i) ? wd : 0.f, step,
-                            1.f, dscale);
+    rc = olmax_adamw_grid(s, master + o, acc + o, mom + o, var + o, shadow + o, n, 0, lr, b1, b2, eps, decays(i) ? wd : 0.f, step,
+                          1.f, dscale, 512, hyper_dev);
     i = j;
   }
   delete[] leaves;
@@ -827,17 +831,19 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
                                           void* params_bf16, const int32_t* ids, const int32_t* labels, float* loss,
                                           void* grad_bf16, float* grad_f32, void* workspace, int64_t workspace_bytes,
                                           int64_t step, float lr, float b1, float b2, float eps, float wd,
-                                          const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch) {
+                                          const int32_t* leaf_decay, float max_grad_norm, float* norm_scratch,
+                                          const float* hyper_dev) {
   RC(check_cfg(c));
   OLMAX_CHECK(master && mom && var && params_bf16 && grad_bf16 && grad_f32, OLMAX_ERR_ARG, "olmax_model_train_step: null pointer");
-  OLMAX_CHECK(step >= 1, OLMAX_ERR_ARG, "olmax_model_train_step: step is 1-based");
+  OLMAX_CHECK(step >= 1 || hyper_dev, OLMAX_ERR_ARG, "olmax_model_train_step: step is 1-based");
+  if (hyper_dev) step = 1;
   // Without recompute the optimizer would share the GPU with the backward GEMMs only (no
   // forward GEMMs in between), which measured 4 % slower than running it afterwards.
   if (!opt_stream || opt_stream == stream || max_grad_norm > 0.f || !c->checkpoint) {
     RC(model_run(stream, c, windows, cos_tables, sin_tables, params_bf16, ids, labels, loss, grad_bf16, grad_f32, workspace,
                  workspace_bytes, true));
     return olmax_model_adamw(stream, c, master, mom, var, params_bf16, grad_bf16, grad_f32, step, lr, b1, b2, eps, wd,
-                             leaf_decay, max_grad_norm, norm_scratch);
+                             leaf_decay, max_grad_norm, norm_scratch, hyper_dev);
   }
   // one event per thread, created on first use and kept for the life of the process
   static thread_local hipEvent_t ev = nullptr;
@@ -847,7 +853,7 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
   olmax_leaf* leaves = new olmax_leaf[nleaf];
   olmax_model_layout(c, leaves, nleaf);
   OverlapCtx x{stream, opt_stream, ev, leaves, nleaf, master, mom, var, (bf16*)params_bf16, (const bf16*)grad_bf16, grad_f32,
-               step, lr, b1, b2, eps, wd, leaf_decay, 0, {0, 0, 0, 0}, 0};
+               step, lr, b1, b2, eps, wd, leaf_decay, hyper_dev, 0, {0, 0, 0, 0}, 0};
   // the optimizer stream must not run ahead of work already queued on the main stream
   int rc = OLMAX_OK;
   if (hipEventRecord(ev, stream) != hipSuccess || hipStreamWaitEvent(opt_stream, ev, 0) != hipSuccess)

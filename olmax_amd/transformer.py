@@ -354,7 +354,7 @@ class Transformer:
     def train_step(self, ids: torch.Tensor, labels: torch.Tensor, *, step: int, lr: float, b1: float = 0.9,
                    b2: float = 0.999, eps: float = 1e-8, weight_decay: float = 1e-4,
                    no_decay_modules: Optional[Sequence[str]] = None, max_grad_norm: Optional[float] = None,
-                   overlap_optimizer: bool = True) -> torch.Tensor:
+                   overlap_optimizer: bool = True, hyper_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
         """loss + gradients + AdamW in one library call (process_microbatch).  With
         ``overlap_optimizer`` each layer's AdamW runs on a second (default-priority) stream while
         the backward pass continues."""
@@ -371,7 +371,7 @@ class Transformer:
             stream_ptr(), opt, ctypes.byref(self.c), self._windows, self._cos, self._sin, ptr(self.master), ptr(self.m),
             ptr(self.v), ptr(self.params_bf16), ptr(ids), ptr(labels), ptr(self.loss), ptr(self.grad_bf16),
             ptr(self.grad_f32), ptr(ws), i64(ws.numel()), i64(step), f32(lr), f32(b1), f32(b2), f32(eps),
-            f32(weight_decay), self.weight_decay_mask(no_decay_modules), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
+            f32(weight_decay), self.weight_decay_mask(no_decay_modules), f32(max_grad_norm or 0.0), ptr(self.norm_scratch), ptr(hyper_dev)))
         return self.loss
 
     def accumulate_grads(self, mini_step: int) -> None:
@@ -385,7 +385,7 @@ class Transformer:
 
     def adamw_step_accumulated(self, *, step: int, lr: float, b1: float = 0.9, b2: float = 0.999, eps: float = 1e-8,
                                weight_decay: float = 1e-4, no_decay_modules: Optional[Sequence[str]] = None,
-                               max_grad_norm: Optional[float] = None) -> None:
+                               max_grad_norm: Optional[float] = None, hyper_dev: Optional[torch.Tensor] = None) -> None:
         """AdamW (and the optional global-norm clip) on the accumulated mean gradient."""
         if self.m is None:
             self.init_optimizer_state()
@@ -394,7 +394,7 @@ class Transformer:
         check(self._L.olmax_model_adamw_accumulated(
             stream_ptr(), ctypes.byref(self.c), ptr(self.master), ptr(self.m), ptr(self.v), ptr(self.params_bf16),
             ptr(self.grad_acc), i64(step), f32(lr), f32(b1), f32(b2), f32(eps), f32(weight_decay),
-            self.weight_decay_mask(no_decay_modules), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
+            self.weight_decay_mask(no_decay_modules), f32(max_grad_norm or 0.0), ptr(self.norm_scratch), ptr(hyper_dev)))
 
     def init_optimizer_state(self) -> None:
         self.m = torch.zeros(self.num_params, device=self.device, dtype=torch.float32)
@@ -402,10 +402,12 @@ class Transformer:
 
     def adamw_step(self, *, step: int, lr: float, b1: float = 0.9, b2: float = 0.999, eps: float = 1e-8,
                    weight_decay: float = 1e-4, no_decay_modules: Optional[Sequence[str]] = None,
-                   max_grad_norm: Optional[float] = None):
+                   max_grad_norm: Optional[float] = None, hyper_dev: Optional[torch.Tensor] = None):
+        """``hyper_dev``: optional fp32 GPU tensor {lr, 1 - b1^step, 1 - b2^step} that replaces the host
+        ``step`` / ``lr`` (schedules that live on the device)."""
         if self.m is None:
             self.init_optimizer_state()
         check(self._L.olmax_model_adamw(
             stream_ptr(), ctypes.byref(self.c), ptr(self.master), ptr(self.m), ptr(self.v), ptr(self.params_bf16),
             ptr(self.grad_bf16), ptr(self.grad_f32), i64(step), f32(lr), f32(b1), f32(b2), f32(eps), f32(weight_decay),
-            self.weight_decay_mask(no_decay_modules), f32(max_grad_norm or 0.0), ptr(self.norm_scratch)))
+            self.weight_decay_mask(no_decay_modules), f32(max_grad_norm or 0.0), ptr(self.norm_scratch), ptr(hyper_dev)))

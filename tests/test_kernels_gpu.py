@@ -463,3 +463,26 @@ def test_adamw(n, gbf):
     p1 = torch.zeros(8).cuda()
     ops.adamw_(p1, torch.tensor([1., -2., 3., -4., 5., -6., 7., -8.]).cuda(), z.clone(), z.clone(), step=1, lr=0.1, wd=0.0)
     assert (p1.cpu() - torch.tensor([-0.1, 0.1] * 4)).abs().max() < 1e-6
+
+
+def test_adamw_with_device_resident_hyperparameters():
+    """olmax_adamw_dev reads lr and the two bias corrections from device memory (hosts whose schedule
+    and step count are device values): with the same three floats it must equal olmax_adamw bit for bit."""
+    ops = _ops()
+    from olmax_amd import _lib
+    from olmax_amd._lib import f32, i32, i64, ptr, stream_ptr, check
+    say("adamw hyper_dev")
+    n, step, lr, b1, b2 = 5003, 7, 3e-3, 0.9, 0.95
+    gen = torch.Generator().manual_seed(1)
+    p = torch.randn(n, generator=gen); m = torch.randn(n, generator=gen) * 0.01; v = torch.rand(n, generator=gen) * 1e-4
+    g = (torch.randn(n, generator=gen) * 0.1).to(BF)
+    a = [t.clone().cuda() for t in (p, m, v)]
+    b = [t.clone().cuda() for t in (p, m, v)]
+    sa, sb = torch.empty(n, dtype=BF).cuda(), torch.empty(n, dtype=BF).cuda()
+    ops.adamw_(a[0], g.cuda(), a[1], a[2], step=step, lr=lr, b1=b1, b2=b2, eps=1e-8, wd=0.1, shadow=sa)
+    hyper = torch.tensor([lr, 1.0 - b1 ** step, 1.0 - b2 ** step], dtype=torch.float64).to(torch.float32).cuda()
+    check(_lib.load().olmax_adamw_dev(stream_ptr(), ptr(b[0]), ptr(g.cuda()), ptr(b[1]), ptr(b[2]), ptr(sb), i64(n), i32(1),
+                                      f32(b1), f32(b2), f32(1e-8), f32(0.1), ptr(hyper), ptr(None)))
+    torch.cuda.synchronize()
+    for x, y in zip(a + [sa], b + [sb]):
+        assert torch.equal(x, y)
