@@ -480,7 +480,9 @@ def test_adamw_with_device_resident_hyperparameters():
     b = [t.clone().cuda() for t in (p, m, v)]
     sa, sb = torch.empty(n, dtype=BF).cuda(), torch.empty(n, dtype=BF).cuda()
     ops.adamw_(a[0], g.cuda(), a[1], a[2], step=step, lr=lr, b1=b1, b2=b2, eps=1e-8, wd=0.1, shadow=sa)
-    hyper = torch.tensor([lr, 1.0 - b1 ** step, 1.0 - b2 ** step], dtype=torch.float64).to(torch.float32).cuda()
+    # the host path forms 1 - b^t in double from the fp32 values of b1 / b2 and rounds once
+    f = lambda x: float(torch.tensor(x, dtype=torch.float32))
+    hyper = torch.tensor([lr, 1.0 - f(b1) ** step, 1.0 - f(b2) ** step], dtype=torch.float64).to(torch.float32).cuda()
     check(_lib.load().olmax_adamw_dev(stream_ptr(), ptr(b[0]), ptr(g.cuda()), ptr(b[1]), ptr(b[2]), ptr(sb), i64(n), i32(1),
                                       f32(b1), f32(b2), f32(1e-8), f32(0.1), ptr(hyper), ptr(None)))
     torch.cuda.synchronize()

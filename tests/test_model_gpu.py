@@ -199,7 +199,8 @@ def test_weight_decay_mask_takes_any_fnmatch_pattern():
     for mm in (m1, m2):
         mm.grad_bf16.normal_(0, 0.01, generator=torch.Generator(device="cuda").manual_seed(1)); mm.grad_f32.fill_(0.01)
     m1.adamw_step(step=3, lr=0.02, b1=0.9, b2=0.95, weight_decay=0.25, no_decay_modules=pats)
-    hyper = torch.tensor([0.02, 1 - 0.9 ** 3, 1 - 0.95 ** 3], dtype=torch.float64).float().cuda()
+    f = lambda x: float(torch.tensor(x, dtype=torch.float32))  # b1 / b2 reach the library as fp32
+    hyper = torch.tensor([0.02, 1 - f(0.9) ** 3, 1 - f(0.95) ** 3], dtype=torch.float64).float().cuda()
     m2.adamw_step(step=0, lr=0.0, b1=0.9, b2=0.95, weight_decay=0.25, no_decay_modules=pats, hyper_dev=hyper)
     assert torch.equal(m1.master, m2.master) and torch.equal(m1.params_bf16, m2.params_bf16)
     # overlapped (per-layer AdamW on a second stream) == sequential, with the same mask and real gradients
