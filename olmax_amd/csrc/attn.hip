@@ -325,39 +325,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
   }
 }
 
-// delta[b,h,i] = sum_d dO[i,h,d] * O[i,h,d]; one 16-lane group per (token, head)
-__global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict__ O,
-                                                         const bf16* __restrict__ dO,
-                                                         float* __restrict__ delta, int B, int S, int H,
-                                                         int64_t ldo, int64_t lddo) {
-  const int sub = threadIdx.x & 15;
-  const int64_t unit = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
-  if (unit >= (int64_t)B * S * H) return;
-  const int64_t tok = unit / H;
-  const int h = (int)(unit % H);
-  Pack8 a, c;
-  a.u = *reinterpret_cast<const u32x4*>(O + tok * ldo + h * 128 + sub * 8);
-  c.u = *reinterpret_cast<const u32x4*>(dO + tok * lddo + h * 128 + sub * 8);
-  float s = 0.f;
-#pragma unroll
-  for (int e = 0; e < 8; e++) s += bf2f(a.e[e]) * bf2f(c.e[e]);
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-  if (sub == 0) {
-    const int64_t bb = tok / S, i = tok % S;
-    delta[(bb * H + h) * S + i] = s;
-  }
-}
-
 // ---------------------------------------------------------------------------------------
 // dQ.  Same tiling and grid as the forward; K/V tiles stream through LDS.
 // ---------------------------------------------------------------------------------------
 template <bool CAP>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     const bf16* __restrict__ Q, const bf16* __restrict__ K, const bf16* __restrict__ V,
-    const bf16* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ DELTA,
-    bf16* __restrict__ dQ, int S, int H, int KH, int64_t ldq, int64_t ldk, int64_t ldv, int64_t lddo,
-    int64_t lddq, float scale, int window, float cap) {
+    const bf16* __restrict__ O, const bf16* __restrict__ dO, const float* __restrict__ LSE,
+    float* __restrict__ DELTA, bf16* __restrict__ dQ, int S, int H, int KH, int64_t ldq, int64_t ldk,
+    int64_t ldv, int64_t ldo, int64_t lddo, int64_t lddq, float scale, int window, float cap) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform for the compiler too
@@ -373,17 +349,26 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
   const int qic = min(qi, S - 1);
 
   bf16x8 qf[8], dof[8];
+  // delta[b,h,i] = sum_d dO[i,h,d] * O[i,h,d]: the two lanes of a query each hold half of its dO
+  // row already, so the row sum costs one pass over O here; it is also written out for the dK/dV
+  // kernel, which runs after this one.
+  float dlt = 0.f;
   {
     const bf16* qp = Q + ((int64_t)b * S + qic) * ldq + h * 128 + lhi * 8;
     const bf16* dp = dO + ((int64_t)b * S + qic) * lddo + h * 128 + lhi * 8;
+    const bf16* op = O + ((int64_t)b * S + qic) * ldo + h * 128 + lhi * 8;
 #pragma unroll
     for (int s = 0; s < 8; s++) {
       qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
       dof[s] = *reinterpret_cast<const bf16x8*>(dp + s * 16);
+      const bf16x8 of = *reinterpret_cast<const bf16x8*>(op + s * 16);
+#pragma unroll
+      for (int e = 0; e < 8; e++) dlt += bf2f(of[e]) * bf2f(dof[s][e]);
     }
   }
+  dlt = half_swap_sum(dlt);
+  if (lhi == 0 && qi < S) DELTA[((int64_t)b * H + h) * S + qi] = dlt;
   const float lse2 = LSE[((int64_t)b * H + h) * S + qic] * LOG2E;
-  const float dlt = DELTA[((int64_t)b * H + h) * S + qic];
   const int j_lo = window >= 0 ? max(0, i0 - window) : 0;
   const int t_lo = j_lo >> 6;
   const int t_hi = min(i0 + 127, S - 1) >> 6;
@@ -784,15 +769,14 @@ bool bwd_fast_ok(const void* q, const void* k, const void* v, const void* o, con
          lddo % 8 == 0 && lddq % 8 == 0 && lddk % 8 == 0 && lddv % 8 == 0;
 }
 
-// The three MFMA kernels of the backward pass (head_dim 128); delta: fp32 [B, H, S] scratch, fully
-// written by the first kernel before the other two read it.
+// The two MFMA kernels of the backward pass (head_dim 128); delta: fp32 [B, H, S] scratch, fully
+// written by the dQ kernel (each workgroup computes the entries of its own queries) before the
+// dK/dV kernel, launched after it, reads them.
 void launch_bwd_fast(hipStream_t stream, const bf16* qp, const bf16* kp, const bf16* vp, const bf16* op, const float* lse,
                      const bf16* gop, bf16* dq, bf16* dk, bf16* dv, float* delta, int B, int S, int H, int KH, int64_t ldq,
                      int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo, int64_t lddq, int64_t lddk, int64_t lddv, int window,
                      float softcap) {
   const float scale = 1.f / sqrtf(128.f);
-  const int64_t units = (int64_t)B * S * H;
-  hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((units + 15) / 16)), dim3(256), 0, stream, op, gop, delta, B, S, H, ldo, lddo);
   dim3 gkv((unsigned)(((S + 127) / 128) * KH * B)), gq((unsigned)(((S + 127) / 128) * H * B));
   constexpr int SM_KV = 2 * (2 * 32 * 256 + 256) + 128 * 256;
   static std::once_flag once;
@@ -803,11 +787,11 @@ void launch_bwd_fast(hipStream_t stream, const bf16* qp, const bf16* kp, const b
     (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
   });
   if (softcap > 0.f) {
+    hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, gq, dim3(256), 65536, stream, qp, kp, vp, op, gop, lse, delta, dq, S, H, KH, ldq, ldk, ldv, ldo, lddo, lddq, scale, window, softcap);
     hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, gkv, dim3(256), SM_KV, stream, qp, kp, vp, gop, lse, delta, dk, dv, S, H, KH, ldq, ldk, ldv, lddo, lddk, lddv, scale, window, softcap);
-    hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, gq, dim3(256), 65536, stream, qp, kp, vp, gop, lse, delta, dq, S, H, KH, ldq, ldk, ldv, lddo, lddq, scale, window, softcap);
   } else {
+    hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, gq, dim3(256), 65536, stream, qp, kp, vp, op, gop, lse, delta, dq, S, H, KH, ldq, ldk, ldv, ldo, lddo, lddq, scale, window, softcap);
     hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, gkv, dim3(256), SM_KV, stream, qp, kp, vp, gop, lse, delta, dk, dv, S, H, KH, ldq, ldk, ldv, lddo, lddk, lddv, scale, window, softcap);
-    hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, gq, dim3(256), 65536, stream, qp, kp, vp, gop, lse, delta, dq, S, H, KH, ldq, ldk, ldv, lddo, lddq, scale, window, softcap);
   }
 }
 
@@ -895,7 +879,7 @@ extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void*
 // instead of a caller-provided workspace.  Each GPU the library runs on holds its own copy of the
 // array (4 MiB) until the process ends; every call on a GPU shares it, so calls that overlap on
 // one GPU (two streams, two threads) race on it.  Nothing in it has to start at zero: the first
-// kernel of a call writes every delta entry the other two read.
+// kernel of a call writes every delta entry the second one reads.
 // ---------------------------------------------------------------------------------------
 constexpr int64_t ATTN_SCRATCH_FLOATS = 1 << 20;  // B * H * S <= 1 Mi (4 MiB)
 static __device__ __align__(256) float scratch[ATTN_SCRATCH_FLOATS];

@@ -5,11 +5,11 @@
 // gradient but still counts in the denominator), fed by LMHead.forward,
 // src/olmax/nn/lm_head.py:59-61 (logits = bf16 GEMM output widened to fp32).
 //
-// One 256-thread block owns one row of logits: pass 1 streams the row with 128-bit loads
-// keeping an online (max, sum-exp) per lane and reduces with wave shuffles; pass 2 re-reads
-// the row (L2-resident: a 100k-entry bf16 row is 200 KB) and overwrites it with
-// d logits = (softmax - onehot) * dloss / n_counted.  Optional final-logit soft-cap
-// z = c*tanh(x/c) is applied on the fly in both passes.
+// One block owns one row of logits.  bf16 rows of up to 163840 entries are loaded ONCE into the
+// block's registers (128-bit loads), reduced to max and sum-exp, and written back as
+// d logits = (softmax - onehot) * dloss / n_counted from the registers; longer or fp32 rows take
+// the streaming form (online max / sum-exp in pass 1, a second read of the row in pass 2).
+// Optional final-logit soft-cap z = c*tanh(x/c) is applied on the fly in both passes.
 #include "common.h"
 
 extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void* B, void* C,
@@ -152,6 +152,81 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
   }
 }
 
+// The same row computation for bf16 rows short enough to keep in registers between the two
+// passes (THREADS x MAXV vectors of 8): the logits are read from memory once and the gradient
+// written once, 4 B per logit instead of 6.  Max and sum-exp are two plain block reductions (no
+// online rescaling needed when the whole row is at hand).
+template <bool CAP, int THREADS, int MAXV>
+__global__ __launch_bounds__(THREADS) void ce_row_regs_kernel(
+    const bf16* __restrict__ logits, bf16* __restrict__ dlogits, const int32_t* __restrict__ labels,
+    float* __restrict__ row_loss, float* __restrict__ lse_out, const int32_t* __restrict__ n_counted,
+    int V, int64_t ld, int64_t ldd, int32_t ignore_index, float cap, float dloss) {
+  constexpr int NW = THREADS / 64;
+  __shared__ float red[NW];
+  const int64_t row = blockIdx.x;
+  const bf16* zr = logits + row * ld;
+  const int label = labels[row];
+  const float inv_cap = CAP ? 1.f / cap : 0.f;
+  const int nvec = V / 8;
+  Pack8 c[MAXV];
+#pragma unroll
+  for (int i = 0; i < MAXV; i++) {
+    const int idx = i * THREADS + threadIdx.x;
+    if (idx < nvec) c[i].u = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(zr) + idx);
+  }
+  auto value = [&](bf16 x) {
+    const float f = bf2f(x);
+    return CAP ? cap * tanhf(f * inv_cap) : f;
+  };
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < MAXV; i++)
+    if (i * THREADS + threadIdx.x < nvec) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) mx = fmaxf(mx, value(c[i].e[e]));
+    }
+  const float gmx = block_max<NW>(mx, red);
+  float sm = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAXV; i++)
+    if (i * THREADS + threadIdx.x < nvec) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) sm += __expf(value(c[i].e[e]) - gmx);
+    }
+  const float gsm = block_sum<NW>(sm, red);
+  const float lse = gmx + __logf(gsm);
+  const bool counted = label != ignore_index;
+  const bool inrange = label >= 0 && label < V;
+  if (threadIdx.x == 0) {
+    const float zl = (counted && inrange) ? value(zr[label]) : 0.f;
+    row_loss[row] = (counted && inrange) ? (lse - zl) : 0.f;
+    if (lse_out) lse_out[row] = counted ? lse : 0.f;
+  }
+  if (!dlogits) return;
+  bf16* dr = dlogits + row * ldd;
+  const float scale = (counted && inrange) ? dloss / (float)(*n_counted) : 0.f;
+#pragma unroll
+  for (int i = 0; i < MAXV; i++) {
+    const int idx = i * THREADS + threadIdx.x;
+    if (idx < nvec) {
+      Pack8 o;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        float z = bf2f(c[i].e[e]), chain = 1.f;
+        if (CAP) {
+          const float t = tanhf(z * inv_cap);
+          z = cap * t;
+          chain = 1.f - t * t;
+        }
+        float p = __expf(z - lse);
+        if (idx * 8 + e == label) p -= 1.f;
+        o.e[e] = f2bf(p * scale * chain);
+      }
+      *(reinterpret_cast<u32x4*>(dr) + idx) = o.u;
+    }
+  }
+}
+
 // loss = sum(row_loss) / n_counted   (single block; deterministic order)
 __global__ __launch_bounds__(256) void ce_finalize_kernel(const float* __restrict__ row_loss, int64_t T,
                                                           const int32_t* __restrict__ n_counted,
@@ -191,12 +266,21 @@ extern "C" int32_t olmax_cross_entropy(hipStream_t stream, const void* logits, v
   hipLaunchKernelGGL((ce_row_kernel<TY, CAPV>), grid, dim3(256), 0, stream, (const TY*)logits,   \
                      (TY*)dlogits, labels, row_loss, lse_out, n_counted, T, V, ld, ldd,          \
                      ignore_index, softcap, dloss, vec_ok)
+#define CE_REGS(CAPV, TH, MV)                                                                              \
+  hipLaunchKernelGGL((ce_row_regs_kernel<CAPV, TH, MV>), grid, dim3(TH), 0, stream, (const bf16*)logits,   \
+                     (bf16*)dlogits, labels, row_loss, lse_out, n_counted, V, ld, ldd, ignore_index, softcap, dloss)
+  const bool regs_ok = !logits_f32 && vec_ok && V % 8 == 0;
   if (logits_f32) {
     if (cap) CE_GO(float, true); else CE_GO(float, false);
+  } else if (regs_ok && V <= 512 * 8 * 26) {  // up to 106496 logits: 8 waves holding 26 vectors each
+    if (cap) CE_REGS(true, 512, 26); else CE_REGS(false, 512, 26);
+  } else if (regs_ok && V <= 1024 * 8 * 20) {  // up to 163840 logits: 16 waves holding 20 vectors each (128 registers per lane)
+    if (cap) CE_REGS(true, 1024, 20); else CE_REGS(false, 1024, 20);
   } else {
     if (cap) CE_GO(bf16, true); else CE_GO(bf16, false);
   }
 #undef CE_GO
+#undef CE_REGS
   hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(256), 0, stream, row_loss, T, n_counted, loss);
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;

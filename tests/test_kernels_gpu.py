@@ -116,7 +116,7 @@ def test_gemm_rejects_bad_arguments():
         ops.gemm(bfr(4, 5), bfr(4, 5))  # CPU tensors: no fallback
 
 
-@pytest.mark.parametrize("rows,d", [(64, 4096), (37, 256), (130, 128), (16, 5376), (9, 4608), (5, 100), (3, 16)])
+@pytest.mark.parametrize("rows,d", [(64, 4096), (37, 256), (130, 128), (16, 5376), (9, 4608), (5, 100), (3, 16), (4100, 4096), (2500, 128)])
 def test_rmsnorm(rows, d):
     ops = _ops()
     say(f"rmsnorm rows{rows} d{d}")
@@ -128,6 +128,10 @@ def test_rmsnorm(rows, d):
     dx, dw = ops.rms_norm_bwd(x.cuda(), w.cuda(), dy.cuda(), 1e-6)
     wdx, wdw = ref.rms_norm_bwd(x.double(), w.double(), dy.double(), 1e-6)
     check_close(dx, wdx, "dx"); check_close(dw, wdw, "dw")
+    # accumulation into a given dw
+    acc = torch.full((d,), 0.5, device="cuda")
+    ops.rms_norm_bwd(x.cuda(), w.cuda(), dy.cuda(), 1e-6, dw=acc)
+    check_close(acc - 0.5, wdw, "dw accumulated", tol=2e-2)
     dx2, _ = ops.rms_norm_bwd(x.cuda(), w.cuda(), dy.cuda(), 1e-6, dres=dres.cuda())
     check_close(dx2, wdx + dres.double(), "dx+dres")
     # no weight
@@ -366,7 +370,8 @@ def test_attention_bwd_on_unaligned_views_stays_inside_its_workspace():
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("T,V,f32", [(33, 4096, False), (17, 1000, True), (8, 50, False), (5, 100352, False)])
+@pytest.mark.parametrize("T,V,f32", [(33, 4096, False), (17, 1000, True), (8, 50, False), (5, 100352, False), (3, 128256, False),
+                                     (3, 262144, False), (6, 1003, False), (4, 4104, True)])
 @pytest.mark.parametrize("cap", [0.0, 30.0])
 def test_cross_entropy(T, V, f32, cap):
     ops = _ops()
