@@ -164,7 +164,9 @@ int32_t olmax_cross_entropy(olmax_stream_t stream, const void* logits, void* dlo
                             int64_t workspace_bytes, int64_t T, int32_t V, int64_t ld, int64_t ldd,
                             int32_t logits_f32, int32_t ignore_index, float softcap, float dloss);
 
-/* ---- Fused LM head + cross entropy, forward and backward: LMHead.forward,
+/* ---- LM head + cross entropy, forward and backward in one call (three GEMMs around a row kernel;
+ * the bf16 logits [T, V] are materialised once in the workspace and overwritten by their gradient,
+ * never as fp32 and never twice): LMHead.forward,
  * src/olmax/nn/lm_head.py:59-61, followed by cross_entropy_loss as in the benchmark's
  * loss_fun, src/integration_tests/train_transformer.py:190-206.
  * dh / dW may be NULL to skip.  dw_f32 != 0: dW is fp32. */

@@ -8,15 +8,21 @@ The reference (epwalsh/OLMax) is pure JAX/Equinox and cannot be imported where t
 runs, and its backward pass is never written down (it comes from
 ``eqx.filter_value_and_grad``, src/olmax/train/trainer.py:734).  Every function here
 therefore restates a reference forward from the cited file:line in plain torch-CPU
-arithmetic and gives a hand-derived backward.  ``tests/test_oracle.py`` pins each one:
-backward formulas against ``torch.autograd`` and finite differences, forwards against
-closed forms, textbook routines (``torch.nn.functional``, ``scipy``) and invariants.
+arithmetic and gives a hand-derived backward.  ``tests/test_oracle.py`` pins each one
+with something that does not share its formula: backward formulas against
+``torch.autograd``, forwards against closed forms, textbook routines
+(``torch.nn.functional``, ``scipy``, ``torch.optim.AdamW``), hand-computed examples and
+invariants; the three block orderings against a block rebuilt from torch's own routines;
+``train_step`` / ``train_batch`` (micro-batch running mean, global-norm clip, masked
+decay) against autograd of the mean loss plus a hand-computed clip factor plus
+``torch.optim.AdamW``; the fp32 RoPE table against the closed form by an ulp bound.
 
-Parity status (what no reference-held vector covers — the reference's tests hold no
-numeric vectors for these ops): attention window off-by-one and the tanh-GELU default
-follow upstream JAX documentation ("parity unpinned" by reference fixtures, pinned by
-brute force / closed forms here); soft-caps, tied embeddings and per-layer windows have
-no reference implementation at all.
+Parity status: every function below has such a check.  What no check here can reach
+(the reference's tests hold no numeric vectors for these ops, and JAX / optax cannot be
+imported): the attention window off-by-one, the tanh-GELU default, optax's epsilon
+placement and MultiSteps averaging follow upstream documentation ("parity unpinned" by
+reference fixtures); soft-caps, tied embeddings and per-layer windows have no reference
+implementation at all.
 
 Rounding model: ``rt`` ("round to") is applied exactly where the reference's bf16 compute
 path rounds (every op output is an array of the compute dtype).  With ``rt=None`` the
