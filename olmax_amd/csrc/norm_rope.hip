@@ -89,6 +89,8 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_generic(const bf16* __restric
 // ------------------------------------------------------------------ RMSNorm backward
 // dx = r*g - x * r^3 * mean(x*g), g = w*dy;   dw[c] += sum_rows dy*x*r   (fp32 atomics)
 // Optional `dres` is added to dx (fused residual-gradient add).
+// Narrow rows (d <= 1024): LPR lanes of one wave own a row, which stays in registers between the
+// two passes, and the lanes' columns sums live in registers until the end.
 template <int LPR, int MAXC, int THREADS>
 __global__ __launch_bounds__(THREADS) void rmsnorm_bwd_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ w, const bf16* __restrict__ dy,
@@ -163,6 +165,147 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_bwd_kernel(
         for (int i = 0; i < MAXC; i++)
           if ((i * LPR + sub) * 8 < d) {
             float* dst = &sdw[(i * LPR + sub) * 8];
+            f32x4 lo, hi;
+            if (turn == 0) {
+#pragma unroll
+              for (int e = 0; e < 4; e++) { lo[e] = dwacc[i][e]; hi[e] = dwacc[i][4 + e]; }
+            } else {
+              lo = *reinterpret_cast<f32x4*>(dst);
+              hi = *reinterpret_cast<f32x4*>(dst + 4);
+#pragma unroll
+              for (int e = 0; e < 4; e++) { lo[e] += dwacc[i][e]; hi[e] += dwacc[i][4 + e]; }
+            }
+            *reinterpret_cast<f32x4*>(dst) = lo;
+            *reinterpret_cast<f32x4*>(dst + 4) = hi;
+          }
+      }
+      __syncthreads();
+    }
+    for (int i = threadIdx.x; i < d; i += THREADS) atomicAdd(&dw[i], sdw[i]);
+  }
+}
+
+// Wide rows (2048 < d <= 8192).  WPR waves share one row, a lane owns MAXC chunks of 8 columns,
+// so the row held between the two passes and the dw column sums take 12 * MAXC registers
+// instead of 128 + 64: sixteen waves fit on a CU, and for a kernel that only streams, waves in
+// flight are what sets the bandwidth.  The waves of a row exchange their partial sums through
+// LDS (two slots used in turn, one barrier per iteration); the next row's x, dy and dres are
+// already on their way while the current one is reduced.
+template <int WPR, int MAXC, int THREADS>
+__global__ __launch_bounds__(THREADS) void rmsnorm_bwd_split_kernel(
+    const bf16* __restrict__ x, const bf16* __restrict__ w, const bf16* __restrict__ dy,
+    const bf16* __restrict__ dres, bf16* __restrict__ dx, float* __restrict__ dw, int64_t rows,
+    int d, int64_t ldx, int64_t lddy, int64_t lddres, int64_t lddx, float eps) {
+  constexpr int RPB = THREADS / (64 * WPR);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rloc = wave / WPR, part = wave % WPR;
+  __shared__ float red[2][RPB][WPR][2];
+  extern __shared__ float sdw[];  // d floats when dw is asked for
+
+  int col[MAXC];
+  bool on[MAXC];
+  Pack8 wv[MAXC];
+  float dwacc[MAXC][8];
+#pragma unroll
+  for (int i = 0; i < MAXC; i++) {
+    col[i] = ((i * WPR + part) * 64 + lane) * 8;
+    on[i] = col[i] < d;
+    wv[i].u = {0u, 0u, 0u, 0u};  // lanes past the end of the row contribute exact zeros
+    if (w && on[i]) wv[i].u = *reinterpret_cast<const u32x4*>(w + col[i]);
+#pragma unroll
+    for (int e = 0; e < 8; e++) dwacc[i][e] = 0.f;
+  }
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  Pack8 nx[MAXC], ng[MAXC], nr[MAXC];
+  auto fetch = [&](int64_t row) {
+    if (row < rows) {
+#pragma unroll
+      for (int i = 0; i < MAXC; i++)
+        if (on[i]) {
+          nx[i].u = *reinterpret_cast<const u32x4*>(x + row * ldx + col[i]);
+          ng[i].u = *reinterpret_cast<const u32x4*>(dy + row * lddy + col[i]);
+          if (dres) nr[i].u = *reinterpret_cast<const u32x4*>(dres + row * lddres + col[i]);
+        }
+    }
+  };
+  const int64_t step = (int64_t)gridDim.x * RPB;
+  int64_t base = (int64_t)blockIdx.x * RPB;
+  fetch(base + rloc);
+  int buf = 0;
+  for (; base < rows; base += step, buf ^= 1) {
+    const int64_t row = base + rloc;
+    Pack8 cx[MAXC], cg[MAXC], cr[MAXC];
+#pragma unroll
+    for (int i = 0; i < MAXC; i++) {
+      cx[i].u = on[i] ? nx[i].u : zero4;
+      cg[i].u = on[i] ? ng[i].u : zero4;
+      cr[i].u = nr[i].u;
+    }
+    fetch(row + step);
+    float ss = 0.f, sxg = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXC; i++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float xf = bf2f(cx[i].e[e]);
+        const float g = w ? bf2f(wv[i].e[e]) * bf2f(cg[i].e[e]) : bf2f(cg[i].e[e]);
+        ss += xf * xf;
+        sxg += xf * g;
+      }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      ss += __shfl_xor(ss, o, 64);
+      sxg += __shfl_xor(sxg, o, 64);
+    }
+    if (lane == 0) {
+      red[buf][rloc][part][0] = ss;
+      red[buf][rloc][part][1] = sxg;
+    }
+    __syncthreads();
+    // Keep the row packed across the barrier: without this the compiler carries the widened
+    // floats of the first pass into the second and doubles the register count.
+#pragma unroll
+    for (int i = 0; i < MAXC; i++) {
+      asm volatile("" : "+v"(cx[i].u), "+v"(cg[i].u), "+v"(wv[i].u));
+    }
+    ss = 0.f;
+    sxg = 0.f;
+#pragma unroll
+    for (int p = 0; p < WPR; p++) {
+      ss += red[buf][rloc][p][0];
+      sxg += red[buf][rloc][p][1];
+    }
+    if (row < rows) {
+      const float r = rsqrtf(ss / (float)d + eps);
+      const float coef = r * r * r * (sxg / (float)d);
+#pragma unroll
+      for (int i = 0; i < MAXC; i++)
+        if (on[i]) {
+          Pack8 o;
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const float xf = bf2f(cx[i].e[e]);
+            const float dyf = bf2f(cg[i].e[e]);
+            const float g = w ? bf2f(wv[i].e[e]) * dyf : dyf;
+            float v = r * g - xf * coef;
+            if (dres) v = bf2f(f2bf(v)) + bf2f(cr[i].e[e]);  // the reference adds two bf16 arrays
+            o.e[e] = f2bf(v);
+            dwacc[i][e] += dyf * xf * r;
+          }
+          *reinterpret_cast<u32x4*>(dx + row * lddx + col[i]) = o.u;
+        }
+    }
+  }
+  if (dw) {
+    // The RPB row slots of the block add their column sums in LDS in turn (every column has one
+    // owner per slot), then one global atomic per column and block.
+#pragma unroll 1
+    for (int turn = 0; turn < RPB; turn++) {
+      if (rloc == turn) {
+#pragma unroll
+        for (int i = 0; i < MAXC; i++)
+          if (on[i]) {
+            float* dst = &sdw[col[i]];
             f32x4 lo, hi;
             if (turn == 0) {
 #pragma unroll
@@ -496,17 +639,21 @@ extern "C" int32_t olmax_rmsnorm_bwd(hipStream_t stream, const void* x, const vo
   const bf16 *xp = (const bf16*)x, *wp = (const bf16*)w, *dyp = (const bf16*)dy, *drp = (const bf16*)dres;
   bf16* dxp = (bf16*)dx;
   const size_t smem = dw ? (size_t)d * 4 : 0;
+#define OLMAX_NORM_BWD_ARGS smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps
   if (vec && d % 8 == 0 && d <= 256) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<16, 2, 256>), dim3(grid_for(rows, 16, 256)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<16, 2, 256>), dim3(grid_for(rows, 16, 256)), dim3(256), OLMAX_NORM_BWD_ARGS);
+  } else if (vec && d % 8 == 0 && d <= 1024) {
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 2, 512>), dim3(grid_for(rows, 8, 256)), dim3(512), OLMAX_NORM_BWD_ARGS);
+  } else if (vec && d % 8 == 0 && d <= 2048) {
+    hipLaunchKernelGGL((rmsnorm_bwd_split_kernel<2, 2, 1024>), dim3(grid_for(rows, 8, 256)), dim3(1024), OLMAX_NORM_BWD_ARGS);
   } else if (vec && d % 8 == 0 && d <= 4096) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 8, 512>), dim3(grid_for(rows, 8, 256)), dim3(512), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
-  } else if (vec && d % 8 == 0 && d <= 6144) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 12, 512>), dim3(grid_for(rows, 8, 256)), dim3(512), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+    hipLaunchKernelGGL((rmsnorm_bwd_split_kernel<4, 2, 1024>), dim3(grid_for(rows, 4, 256)), dim3(1024), OLMAX_NORM_BWD_ARGS);
   } else if (vec && d % 8 == 0 && d <= 8192) {
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<64, 16, 256>), dim3(grid_for(rows, 4, 256)), dim3(256), smem, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
+    hipLaunchKernelGGL((rmsnorm_bwd_split_kernel<8, 2, 1024>), dim3(grid_for(rows, 2, 256)), dim3(1024), OLMAX_NORM_BWD_ARGS);
   } else {
     hipLaunchKernelGGL(rmsnorm_bwd_generic, dim3(grid_for(rows, 1, 1 << 16)), dim3(256), 0, stream, xp, wp, dyp, drp, dxp, dw, rows, d, ldx, lddy, lddres, lddx, eps);
   }
+#undef OLMAX_NORM_BWD_ARGS
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
 }

@@ -116,7 +116,8 @@ def test_gemm_rejects_bad_arguments():
         ops.gemm(bfr(4, 5), bfr(4, 5))  # CPU tensors: no fallback
 
 
-@pytest.mark.parametrize("rows,d", [(64, 4096), (37, 256), (130, 128), (16, 5376), (9, 4608), (5, 100), (3, 16), (4100, 4096), (2500, 128)])
+@pytest.mark.parametrize("rows,d", [(64, 4096), (37, 256), (130, 128), (16, 5376), (9, 4608), (5, 100), (3, 16), (4100, 4096), (2500, 128),
+                                    (300, 3080), (1030, 2056), (77, 1032), (519, 2048), (40, 1024), (1025, 8192), (33, 6152), (7, 264)])
 def test_rmsnorm(rows, d):
     ops = _ops()
     say(f"rmsnorm rows{rows} d{d}")
