@@ -434,3 +434,52 @@ def test_fit_loop_logs_every_step_once_with_losses_of_a_manual_run():
         assert m["optim/g_norm"] == pytest.approx(gn, rel=2e-2)
         assert m["throughput/TPS"] == pytest.approx(m["throughput/BPS"] * 2 * B * S)
         assert ("throughput/TPS average" in m) == (s >= 10)
+
+
+@pytest.mark.parametrize("overlap", [False, True])
+def test_train_step_captured_in_a_hip_graph_replays_like_eager_steps(overlap):
+    """The library only enqueues on the streams it is handed (zeroing is a fill kernel, the
+    optimizer stream is forked and joined with events inside the call), so one train step can be
+    recorded into a HIP graph once and replayed: with the token buffers and the three
+    step-dependent scalars {lr, 1 - b1^t, 1 - b2^t} updated in place between replays, four
+    replays must walk the same losses and parameters as four eager calls.  Every replay is
+    checked, with eager copies and a synchronisation between replays."""
+    say(f"train step under graph capture, overlap={overlap}")
+    ocfg, hcfg = _cfgs("gemma")
+    hcfg.layer_ac_policy = "nothing_saveable"
+    B, S, steps = 2, 128, 5
+    P = _params(ocfg)
+    b1, b2 = 0.9, 0.95
+    f = lambda x: float(torch.tensor(x, dtype=torch.float32))
+    batches, hypers = [], []
+    for t in range(1, steps + 1):
+        gen = torch.Generator().manual_seed(100 + t)
+        batches.append((torch.randint(0, 512, (B * S,), generator=gen, dtype=torch.int32).cuda(),
+                        torch.randint(0, 512, (B * S,), generator=gen, dtype=torch.int32).cuda()))
+        lr = 1e-3 * t  # a schedule that moves every step
+        hypers.append(torch.tensor([lr, 1 - f(b1) ** t, 1 - f(b2) ** t], dtype=torch.float64).float().cuda())
+    kw = dict(step=0, lr=0.0, b1=b1, b2=b2, weight_decay=0.1, overlap_optimizer=overlap)
+
+    eager = hcfg.build(batch_size=B, sequence_length=S); eager.load_state_dict(P)
+    want = []
+    for (ids, labels), hy in zip(batches, hypers):
+        loss = eager.train_step(ids, labels, hyper_dev=hy, **kw)
+        want.append((loss.item(), eager.master.clone()))
+
+    model = hcfg.build(batch_size=B, sequence_length=S); model.load_state_dict(P)
+    ids_buf, labels_buf, hyper_buf = batches[0][0].clone(), batches[0][1].clone(), hypers[0].clone()
+    # step 1 eagerly (kernel attributes, workspace and optimizer state exist before the capture starts)
+    loss = model.train_step(ids_buf, labels_buf, hyper_dev=hyper_buf, **kw)
+    assert loss.item() == pytest.approx(want[0][0], rel=1e-5)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        model.train_step(ids_buf, labels_buf, hyper_dev=hyper_buf, **kw)
+    assert relerr(model.master, want[0][1]) < 1e-6  # recording ran nothing
+    for t in range(1, steps):
+        ids_buf.copy_(batches[t][0]); labels_buf.copy_(batches[t][1]); hyper_buf.copy_(hypers[t])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert model.loss.item() == pytest.approx(want[t][0], rel=1e-5), t
+        assert relerr(model.master, want[t][1]) < 1e-5, t
+        assert torch.equal(model.params_bf16, model.master.to(BF)), t
