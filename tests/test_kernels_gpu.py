@@ -83,12 +83,13 @@ def test_gemm_brute_force_tiny_and_strided():
 
 
 @pytest.mark.parametrize("al,bl", [(0, 0), (0, 1), (1, 1), (1, 0)])
-@pytest.mark.parametrize("M,N,K", [(2048, 4096, 192), (2048, 4096, 256), (4096, 4352, 64)])
+@pytest.mark.parametrize("M,N,K", [(2048, 4096, 192), (2048, 4096, 256), (4096, 4352, 64), (4096, 8448, 256), (4096, 12288, 384)])
 def test_gemm_256_tiles_row_strided_operands(M, N, K, al, bl):
     """The 256x256-tile kernel (>= 128 tiles) with every operand a column slice of a wider buffer
     (leading dimensions that are not the row length, 16-byte aligned offsets), odd and even k-tile
     counts, a strided residual and a strided output; the 272-tile case is cut into whole rounds
-    plus a remainder.  Against a float64 product of the same bf16 values."""
+    plus a remainder; the 528- and 768-tile cases have more tiles than the GPU has CUs (two and
+    three rounds of workgroups).  Against a float64 product of the same bf16 values."""
     ops = _ops()
     say(f"gemm 256-tile strided M{M} N{N} K{K} a{al} b{bl}")
     ar, ac = (M, K) if al == 0 else (K, M)
