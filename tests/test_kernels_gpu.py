@@ -495,3 +495,65 @@ def test_adamw_with_device_resident_hyperparameters():
     torch.cuda.synchronize()
     for x, y in zip(a + [sa], b + [sb]):
         assert torch.equal(x, y)
+
+
+def test_two_host_threads_on_their_own_streams_get_single_thread_results():
+    """The entry points are re-entrant: they enqueue on the stream they are given, keep no
+    per-call state outside their arguments and report errors through a thread-local string.
+    Two host threads (ctypes releases the GIL during a call) each drive GEMM, RMSNorm and the
+    attention forward / backward on a stream of their own, 25 rounds; every result must be
+    bit-identical to the one the same inputs give from a single thread (these kernels use no
+    atomics), and an argument error raised in one thread must not show up in the other."""
+    import threading
+    ops = _ops()
+    from olmax_amd import _lib
+    say("two host threads, two streams")
+    B, S, H, KH, D = 1, 512, 2, 1, 128
+
+    def inputs(seed):
+        return dict(a=bfr(512, 256, seed=seed).cuda(), b=bfr(768, 256, seed=seed + 1).cuda(),
+                    x=bfr(300, 4096, seed=seed + 2).cuda(), w=bfr(4096, seed=seed + 3).cuda(),
+                    q=bfr(B * S, H * D, seed=seed + 4).cuda(), k=bfr(B * S, KH * D, seed=seed + 5).cuda(),
+                    v=bfr(B * S, KH * D, seed=seed + 6).cuda(), do=bfr(B * S, H * D, seed=seed + 7).cuda())
+
+    def work(t):
+        c = ops.gemm(t["a"], t["b"])
+        y = ops.rms_norm_fwd(t["x"], t["w"], 1e-6)
+        o, lse = ops.attn_fwd(t["q"], t["k"], t["v"], B=B, S=S, H=H, KH=KH, D=D)
+        dq, dk, dv = ops.attn_bwd(t["q"], t["k"], t["v"], o, lse, t["do"], B=B, S=S, H=H, KH=KH, D=D)
+        return [c, y, o, lse, dq, dk, dv]
+
+    ins = [inputs(10), inputs(20)]
+    want = [work(t) for t in ins]
+    torch.cuda.synchronize()
+    errors, seen = [], [None, None]
+
+    def run(idx):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for it in range(25):
+                    got = work(ins[idx])
+                    if idx == 0 and it == 5:  # an argument error in this thread only
+                        try:
+                            ops.attn_fwd(ins[0]["q"], ins[0]["k"], ins[0]["v"], B=B, S=S, H=3, KH=2, D=D)
+                        except _lib.OlmaxHipError as e:
+                            seen[0] = str(e)
+                    stream.synchronize()
+                    for g, w_ in zip(got, want[idx]):
+                        if not torch.equal(g, w_):
+                            errors.append((idx, it))
+                if idx == 1:
+                    seen[1] = _lib.load().olmax_last_error_string().decode()
+        except Exception as e:  # noqa: BLE001 - reported below, in the main thread
+            errors.append((idx, repr(e)))
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads)
+    assert not errors, errors
+    assert seen[0], "the bad call in thread 0 must raise"
+    assert seen[1] == "", f"thread 1 saw another thread's error: {seen[1]!r}"
