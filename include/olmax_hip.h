@@ -131,6 +131,9 @@ int32_t olmax_attn_fwd(olmax_stream_t stream, const void* q, const void* k, cons
                        float* lse, int32_t B, int32_t S, int32_t H, int32_t KH, int32_t D, int64_t ldq,
                        int64_t ldk, int64_t ldv, int64_t ldo, int32_t window, float softcap);
 int64_t olmax_attn_bwd_workspace_bytes(int32_t B, int32_t S, int32_t H, int32_t KH, int32_t D);
+/* The part of that size the MFMA path needs (delta, [B, H, S] fp32): enough when head_dim is 128
+ * and every operand is 16-byte aligned with row strides that are multiples of 8. */
+int64_t olmax_attn_bwd_workspace_bytes_aligned(int32_t B, int32_t S, int32_t H);
 int32_t olmax_attn_bwd(olmax_stream_t stream, const void* q, const void* k, const void* v,
                        const void* o, const float* lse, const void* d_o, void* dq, void* dk, void* dv,
                        void* workspace, int64_t workspace_bytes, int32_t B, int32_t S, int32_t H,
@@ -146,7 +149,12 @@ int32_t olmax_attn_bwd(olmax_stream_t stream, const void* q, const void* k, cons
  * aligned with row strides that are multiples of 8, otherwise an error is returned and nothing
  * is launched.  Calls no hipMalloc / hipFree.  All calls on one GPU share the array: calls that
  * overlap on one GPU (different streams or threads) race.  Results equal olmax_attn_bwd's bit for
- * bit (same kernels). */
+ * bit (same kernels).
+ * Set-up: the scratch address is resolved per device by olmax_attn_bwd_noalloc_init() (device
+ * current; no stream work, no allocation) or, failing that, by the first eager call.  Before the
+ * entry point is recorded into a HIP graph one of the two must have happened on that device: a
+ * first use under stream capture returns an error instead of querying the symbol there. */
+int32_t olmax_attn_bwd_noalloc_init(void);
 int64_t olmax_attn_bwd_noalloc_max_rows(void);
 int32_t olmax_attn_bwd_noalloc(olmax_stream_t stream, const void* q, const void* k, const void* v,
                                const void* o, const float* lse, const void* d_o, void* dq, void* dk,
@@ -369,6 +377,10 @@ int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, double*
  * on the calling host thread, visible to rocprofv3 --marker-trace.  Needs a roctx library at run
  * time; returns an error (and stays off) without it. */
 int32_t olmax_set_profiler_ranges(int32_t on);
+/* Number of AdamW launch groups the calling thread's last olmax_model_train_step put on its
+ * optimizer stream; 0 means that step ran AdamW after the backward pass on the main stream
+ * (no second stream, clipping on, or activations kept).  For tests of the overlapped path. */
+int32_t olmax_model_last_step_overlapped_launches(void);
 
 #ifdef __cplusplus
 }

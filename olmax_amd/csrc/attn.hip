@@ -769,6 +769,18 @@ bool bwd_fast_ok(const void* q, const void* k, const void* v, const void* o, con
          lddo % 8 == 0 && lddq % 8 == 0 && lddk % 8 == 0 && lddv % 8 == 0;
 }
 
+constexpr int SM_KV = 2 * (2 * 32 * 256 + 256) + 128 * 256;
+// dynamic-LDS limits of the backward kernels, set once per process
+void bwd_fast_attributes() {
+  static std::once_flag once;
+  std::call_once(once, [] {
+    (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
+    (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
+    (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+  });
+}
+
 // The two MFMA kernels of the backward pass (head_dim 128); delta: fp32 [B, H, S] scratch, fully
 // written by the dQ kernel (each workgroup computes the entries of its own queries) before the
 // dK/dV kernel, launched after it, reads them.
@@ -778,14 +790,7 @@ void launch_bwd_fast(hipStream_t stream, const bf16* qp, const bf16* kp, const b
                      float softcap) {
   const float scale = 1.f / sqrtf(128.f);
   dim3 gkv((unsigned)(((S + 127) / 128) * KH * B)), gq((unsigned)(((S + 127) / 128) * H * B));
-  constexpr int SM_KV = 2 * (2 * 32 * 256 + 256) + 128 * 256;
-  static std::once_flag once;
-  std::call_once(once, [] {
-    (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
-    (void)hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SM_KV);
-    (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-    (void)hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-  });
+  bwd_fast_attributes();
   if (softcap > 0.f) {
     hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, gq, dim3(256), 65536, stream, qp, kp, vp, op, gop, lse, delta, dq, S, H, KH, ldq, ldk, ldv, ldo, lddo, lddq, scale, window, softcap);
     hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, gkv, dim3(256), SM_KV, stream, qp, kp, vp, gop, lse, delta, dk, dv, S, H, KH, ldq, ldk, ldv, lddo, lddk, lddv, scale, window, softcap);
@@ -838,6 +843,9 @@ static int64_t attn_acc_bytes(int32_t B, int32_t S, int32_t KH, int32_t D) { ret
 extern "C" int64_t olmax_attn_bwd_workspace_bytes(int32_t B, int32_t S, int32_t H, int32_t KH, int32_t D) {
   return attn_delta_bytes(B, S, H) + 2 * attn_acc_bytes(B, S, KH, D);
 }
+// What the MFMA path alone needs (delta only): for callers that KNOW head_dim is 128 and every
+// operand is 16-byte aligned with row strides that are multiples of 8.
+extern "C" int64_t olmax_attn_bwd_workspace_bytes_aligned(int32_t B, int32_t S, int32_t H) { return attn_delta_bytes(B, S, H); }
 
 extern "C" int32_t olmax_attn_bwd(hipStream_t stream, const void* q, const void* k, const void* v,
                                   const void* o, const float* lse, const void* d_o, void* dq, void* dk,
@@ -891,12 +899,18 @@ float* g_scratch_ptr[MAX_DEVICES];  // device address of `scratch` on each GPU, 
 
 // The array's name is only a host-side handle; its device address differs per GPU and comes
 // from hipGetSymbolAddress with that GPU current.
-int scratch_for_current_device(float** out) {
+// resolve == false: only look the address up (what a call under graph capture may do); the
+// symbol query itself belongs to set-up, outside any capture.
+int scratch_for_current_device(float** out, bool resolve) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
     return olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_attn_bwd_noalloc: cannot identify the current device");
   std::lock_guard<std::mutex> lock(g_scratch_mu);
   if (!g_scratch_ptr[dev]) {
+    if (!resolve)
+      return olmax_set_error(OLMAX_ERR_ARG,
+                             "olmax_attn_bwd_noalloc: first use on this device is under stream capture; call "
+                             "olmax_attn_bwd_noalloc_init() (or the entry point once, eagerly) before recording");
     float* p = nullptr;
     const hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !p)
@@ -907,6 +921,15 @@ int scratch_for_current_device(float** out) {
   return OLMAX_OK;
 }
 }  // namespace
+
+// Set-up for the current device: resolves the scratch address and sets the kernels' LDS limits.
+// Call it once per device (with that device current) before recording olmax_attn_bwd_noalloc
+// into a graph; an eager call of the entry point does the same.
+extern "C" int32_t olmax_attn_bwd_noalloc_init(void) {
+  float* p = nullptr;
+  bwd_fast_attributes();
+  return scratch_for_current_device(&p, true);
+}
 
 extern "C" int64_t olmax_attn_bwd_noalloc_max_rows(void) { return ATTN_SCRATCH_FLOATS; }
 
@@ -924,7 +947,13 @@ extern "C" int32_t olmax_attn_bwd_noalloc(hipStream_t stream, const void* q, con
   OLMAX_CHECK(bwd_fast_ok(q, k, v, o, d_o, dq, dk, dv, D, ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv), OLMAX_ERR_ALIGN,
               "olmax_attn_bwd_noalloc: needs head_dim 128, 16-byte aligned pointers and row strides that are multiples of 8; use olmax_attn_bwd otherwise");
   float* delta = nullptr;
-  { int rc = scratch_for_current_device(&delta); if (rc) return rc; }
+  {
+    // under capture only a pointer resolved earlier may be used: the symbol query is set-up work
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    const bool capturing = stream && hipStreamIsCapturing(stream, &st) == hipSuccess && st == hipStreamCaptureStatusActive;
+    int rc = scratch_for_current_device(&delta, !capturing);
+    if (rc) return rc;
+  }
   launch_bwd_fast(stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)o, lse, (const bf16*)d_o, (bf16*)dq, (bf16*)dk,
                   (bf16*)dv, delta, B, S, H, KH, ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv, window, softcap);
   OLMAX_LAUNCH_CHECK();

@@ -252,9 +252,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(16))) void adam
   if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
     const int64_t i = n4 * 4 + threadIdx.x;
     const float ge = (G_BF16 ? bf2f(reinterpret_cast<const bf16*>(gv)[i]) : reinterpret_cast<const float*>(gv)[i]) * gscale;
-    const float mm = b1 * m[i] + (1.f - b1) * ge;
-    const float vv = b2 * v[i] + (1.f - b2) * ge * ge;
-    const float pp = p[i] - lr * ((mm / bc1) / (sqrtf(vv / bc2) + eps) + wd * p[i]);
+    // the same operations in the same order as the vector body: where a range is cut does not
+    // change any element's result
+    const float mm = b1 * m[i] + omb1 * ge;
+    const float vv = b2 * v[i] + omb2 * ge * ge;
+    const float mh = mm * ibc1;
+    const float vh = vv * ibc2;
+    const float pp = p[i] - lr * (mh / (sqrtf(vh) + eps) + wd * p[i]);
     m[i] = mm;
     v[i] = vv;
     p[i] = pp;

@@ -71,10 +71,24 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
     int vec_ok) {
   constexpr int VEC = Io<T>::VEC;
   __shared__ float red[4];
+  __shared__ float label_logit;
   const int64_t row = blockIdx.x;
   const T* zr = logits + row * ld;
   const int label = labels[row];
   const float inv_cap = CAP ? 1.f / cap : 0.f;
+  const bool counted = label != ignore_index;
+  const bool inrange = label >= 0 && label < V;
+  // The label's logit is fetched and parked in LDS BEFORE the first block barrier: with dlogits
+  // aliasing logits, other waves overwrite the row as soon as they are past the last reduction,
+  // and no load of the row may be left to race with those stores.
+  if (threadIdx.x == 0) {
+    float zl = 0.f;
+    if (counted && inrange) {
+      zl = Io<T>::ld1(zr + label);
+      if (CAP) zl = cap * tanhf(zl * inv_cap);
+    }
+    label_logit = zl;
+  }
   // ---- pass 1: online max / sum-exp ----
   float mx = -INFINITY, sm = 0.f;
   const int nvec = vec_ok ? V / VEC : 0;
@@ -107,15 +121,8 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
   sm = (mx == -INFINITY) ? 0.f : sm * __expf(mx - gmx);
   const float gsm = block_sum<4>(sm, red);
   const float lse = gmx + __logf(gsm);
-  const bool counted = label != ignore_index;
-  const bool inrange = label >= 0 && label < V;
   if (threadIdx.x == 0) {
-    float zl = 0.f;
-    if (counted && inrange) {
-      zl = Io<T>::ld1(zr + label);
-      if (CAP) zl = cap * tanhf(zl * inv_cap);
-    }
-    row_loss[row] = (counted && inrange) ? (lse - zl) : 0.f;
+    row_loss[row] = (counted && inrange) ? (lse - label_logit) : 0.f;
     if (lse_out) lse_out[row] = counted ? lse : 0.f;
   }
   if (!dlogits) return;
@@ -163,11 +170,24 @@ __global__ __launch_bounds__(THREADS) void ce_row_regs_kernel(
     int V, int64_t ld, int64_t ldd, int32_t ignore_index, float cap, float dloss) {
   constexpr int NW = THREADS / 64;
   __shared__ float red[NW];
+  __shared__ float label_logit;
   const int64_t row = blockIdx.x;
   const bf16* zr = logits + row * ld;
   const int label = labels[row];
   const float inv_cap = CAP ? 1.f / cap : 0.f;
   const int nvec = V / 8;
+  const bool counted = label != ignore_index;
+  const bool inrange = label >= 0 && label < V;
+  // label logit into LDS before the first barrier (see ce_row_kernel): nothing reads the row
+  // from memory once any wave may be storing the gradient over it
+  if (threadIdx.x == 0) {
+    float zl = 0.f;
+    if (counted && inrange) {
+      zl = bf2f(zr[label]);
+      if (CAP) zl = cap * tanhf(zl * inv_cap);
+    }
+    label_logit = zl;
+  }
   Pack8 c[MAXV];
 #pragma unroll
   for (int i = 0; i < MAXV; i++) {
@@ -195,11 +215,8 @@ __global__ __launch_bounds__(THREADS) void ce_row_regs_kernel(
     }
   const float gsm = block_sum<NW>(sm, red);
   const float lse = gmx + __logf(gsm);
-  const bool counted = label != ignore_index;
-  const bool inrange = label >= 0 && label < V;
   if (threadIdx.x == 0) {
-    const float zl = (counted && inrange) ? value(zr[label]) : 0.f;
-    row_loss[row] = (counted && inrange) ? (lse - zl) : 0.f;
+    row_loss[row] = (counted && inrange) ? (lse - label_logit) : 0.f;
     if (lse_out) lse_out[row] = counted ? lse : 0.f;
   }
   if (!dlogits) return;

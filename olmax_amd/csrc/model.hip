@@ -97,7 +97,11 @@ Tmp carve_tmp(const olmax_model_config* c, Arena& a) {
   t.d_o = a.take<bf16>(m.T * m.HD);
   t.dqkv = a.take<bf16>(m.T * m.QKV);
   if (c->qk_norm) t.dqkr = a.take<bf16>(m.T * (m.HD + m.KD));
-  t.attn_ws_bytes = olmax_attn_bwd_workspace_bytes(m.B, m.S, m.H, m.K, m.D);
+  // every buffer of the arena is 256-byte aligned and every row stride a multiple of 8, so head
+  // dim 128 always takes the MFMA path, which needs delta only (the generic path's two fp32
+  // accumulators would be 256 MiB at the 7B shape)
+  t.attn_ws_bytes = m.D == 128 ? olmax_attn_bwd_workspace_bytes_aligned(m.B, m.S, m.H)
+                               : olmax_attn_bwd_workspace_bytes(m.B, m.S, m.H, m.K, m.D);
   t.attn_ws = a.take<char>(t.attn_ws_bytes);
   return t;
 }
@@ -569,6 +573,10 @@ struct OverlapCtx {
   int head_windows = 0;     // windows still to come
   int64_t layer_numel = 0;  // parameters of one layer (the size of a window's own update)
 };
+// AdamW launches the last olmax_model_train_step of this host thread put on its optimizer stream
+// (0: the step took the sequential branch); read back by tests through
+// olmax_model_last_step_overlapped_launches
+thread_local int g_overlapped_launches = 0;
 int overlap_launch(OverlapCtx* x, int layer);
 int overlap_flush(void* vctx, int point) {
   OverlapCtx* x = (OverlapCtx*)vctx;
@@ -592,6 +600,7 @@ int overlap_head_chunk(OverlapCtx* x, int64_t n, int grid_cap) {
   const int64_t o = lf.offset + x->head_done;
   x->head_done += n;
   const float lwd = (!x->leaf_decay || x->leaf_decay[x->head_leaf]) ? x->wd : 0.f;
+  g_overlapped_launches++;
   return olmax_adamw_grid(x->opt, x->master + o, x->G + o, x->mom + o, x->var + o, x->shadow + o, n, 1, x->lr, x->b1, x->b2, x->eps,
                           lwd, x->step, 1.f, nullptr, grid_cap, x->hyper_dev);
 }
@@ -609,6 +618,7 @@ int overlap_launch(OverlapCtx* x, int layer) {
     }
   }
   if (begin < 0) return OLMAX_OK;
+  g_overlapped_launches++;
   if (hipEventRecord(x->ev, x->main) != hipSuccess || hipStreamWaitEvent(x->opt, x->ev, 0) != hipSuccess)
     return olmax_set_error(OLMAX_ERR_LAUNCH, "olmax_model_train_step: event record/wait failed");
   // One workgroup per CU is the grid that disturbs the GEMMs it runs beside least, but alone it only
@@ -875,6 +885,8 @@ extern "C" int32_t olmax_model_adamw_accumulated(hipStream_t s, const olmax_mode
 // concurrently with the backward pass of the layers below it (MFMA-bound); `stream` waits for
 // the optimizer stream before returning control to later work.  Both streams must have the
 // default priority.  opt_stream == NULL (or clipping on) gives the plain sequence.
+extern "C" int32_t olmax_model_last_step_overlapped_launches(void) { return g_overlapped_launches; }
+
 extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_stream, const olmax_model_config* c,
                                           const int32_t* windows, const float* const* cos_tables,
                                           const float* const* sin_tables, float* master, float* mom, float* var,
@@ -887,6 +899,7 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
   OLMAX_CHECK(master && mom && var && params_bf16 && grad_bf16 && grad_f32, OLMAX_ERR_ARG, "olmax_model_train_step: null pointer");
   OLMAX_CHECK(step >= 1 || hyper_dev, OLMAX_ERR_ARG, "olmax_model_train_step: step is 1-based");
   if (hyper_dev) step = 1;
+  g_overlapped_launches = 0;
   // Without recompute the optimizer would share the GPU with the backward GEMMs only (no
   // forward GEMMs in between), which measured 4 % slower than running it afterwards.
   if (!opt_stream || opt_stream == stream || max_grad_norm > 0.f || !c->checkpoint) {

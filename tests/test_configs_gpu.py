@@ -130,16 +130,52 @@ def test_config5_gemma3_slice_full_width_with_adamw():
     ocfg = ref.ModelConfig(vocab=262144, d_model=5376, n_layers=L, n_heads=32, n_kv_heads=16, head_dim=128, hidden=21504,
                            layer_type="gemma", act="gelu", qk_norm=True, eps=1e-6, rope_theta_layers=th, windows=win, tied=True)
     model, loss = _model_prefix_check(hcfg, ocfg, 2, 4096, seed=12)
-    # AdamW step 1 with zero state: |delta p| = lr * |sign(g) + wd p| wherever |g| >> eps
-    leaf = next(l for l in model.leaves if model.leaf_name(l) == "layers.3.mlp.down_proj.weight")
-    sl = slice(leaf.offset, leaf.offset + leaf.numel)
-    before = model.master[sl].clone()
-    model.adamw_step(step=1, lr=1e-3, weight_decay=0.0)
-    delta = (model.master[sl] - before).abs()
-    big = model.grad_bf16[sl].float().abs() > 1e-4
-    assert big.any()
-    assert (delta[big] - 1e-3).abs().max().item() < 2e-5
-    assert torch.equal(model.params_bf16[sl], model.master[sl].to(BF))
+    # The fused AdamW step of this configuration against the oracle (optax.adamw as built at
+    # src/olmax/optim/config.py:136-148): two steps on the gradients just computed, weight decay
+    # on, the embedding and every norm weight masked; master, m, v compared on sampled slices of
+    # three leaves (a matrix with bf16 gradients, a masked norm weight and the masked, tied
+    # embedding, both with fp32 gradients) after the SECOND step (non-zero moments, both bias
+    # corrections != 1).
+    pats = ["embedding.weight", "*norm.weight"]
+    picks = {"layers.3.mlp.down_proj.weight": 0.05, "layers.0.attention.k_proj.weight": 0.05,
+             "layers.4.attention.q_norm.weight": 0.0, "embedding.weight": 0.0}  # leaf -> the decay it must see
+    leaves = {model.leaf_name(l): l for l in model.leaves}
+    G = model.named_gradients()
+    want, before = {}, {}
+    gidx = torch.Generator().manual_seed(5)
+    for n, wd in picks.items():
+        l = leaves[n]
+        idx = torch.randint(0, l.numel, (min(l.numel, 50_000),), generator=gidx).cuda()
+        p = model.master[l.offset: l.offset + l.numel][idx].double().cpu()
+        before[n] = p.clone()
+        g = G[n].reshape(-1)[idx].double().cpu()
+        assert g.abs().max().item() > 0, n
+        m, v = torch.zeros_like(p), torch.zeros_like(p)
+        for step in (1, 2):
+            p, m, v = ref.adamw_step(p, g, m, v, step=step, lr=1e-3, b1=0.9, b2=0.95, eps=1e-8, wd=wd)
+        want[n] = (idx, p, m, v)
+    model.init_optimizer_state()
+    for step in (1, 2):
+        model.adamw_step(step=step, lr=1e-3, b1=0.9, b2=0.95, eps=1e-8, weight_decay=0.05, no_decay_modules=pats)
+    for n, (idx, p, m, v) in want.items():
+        l = leaves[n]
+        sl = slice(l.offset, l.offset + l.numel)
+        # 1e-6 of the leaf's scale: fp32 rounding of p itself; a decay applied to a masked leaf (or left
+        # out of an unmasked one) moves an element by lr * wd * p * 2 = 1e-4 p
+        assert (model.master[sl][idx].double().cpu() - p).abs().max().item() <= 1e-6 * p.abs().max().item(), n
+        assert (model.m[sl][idx].double().cpu() - m).abs().max().item() <= 1e-6 * m.abs().max().item() + 1e-12, n
+        assert (model.v[sl][idx].double().cpu() - v).abs().max().item() <= 1e-6 * v.abs().max().item() + 1e-20, n
+        assert torch.equal(model.params_bf16[sl], model.master[sl].to(BF)), n
+    # the tolerance does tell the two groups apart: the matrix against an oracle run WITHOUT decay misses
+    n = "layers.3.mlp.down_proj.weight"
+    idx, p, _, _ = want[n]
+    l = leaves[n]
+    p0 = before[n]
+    g = G[n].reshape(-1)[idx].double().cpu()
+    m, v = torch.zeros_like(p0), torch.zeros_like(p0)
+    for step in (1, 2):
+        p0, m, v = ref.adamw_step(p0, g, m, v, step=step, lr=1e-3, b1=0.9, b2=0.95, eps=1e-8, wd=0.0)
+    assert (model.master[l.offset: l.offset + l.numel][idx].double().cpu() - p0).abs().max().item() > 1e-6 * p.abs().max().item()
 
 
 def test_config3_llama7b_full_model():
@@ -170,6 +206,40 @@ def test_config3_llama7b_full_model():
     emb = model.named_parameters()["embedding.weight"]
     ws_rows = model.workspace().view(torch.bfloat16)[: 4 * cfg.d_model].view(4, cfg.d_model)
     assert torch.equal(ws_rows, emb[ids[:4].long()].to(BF))
+
+    # The step the benchmark times (second stream, full-block recompute, LM-head update cut into 32
+    # pieces) against the sequential step, from the same seeded state: integer checksums of the
+    # bit patterns of master / m / v / bf16 copy over the LM head and three layers must be equal
+    # (AdamW is elementwise, the bf16 gradients are deterministic).
+    from olmax_amd import _lib
+    model.c.checkpoint = 1
+    model._workspace = None
+    torch.cuda.empty_cache()
+    leaves = {model.leaf_name(l): l for l in model.leaves}
+    spans = {"lm_head": (leaves["lm_head.proj.weight"].offset, leaves["lm_head.proj.weight"].numel)}
+    for l in (0, 15, 31):
+        first, last = leaves[f"layers.{l}.attention.q_proj.weight"], leaves[f"layers.{l}.mlp.down_proj.weight"]
+        spans[f"layer{l}"] = (first.offset, last.offset + last.numel - first.offset)
+
+    def checksums():
+        out = {}
+        for k, (o, n) in spans.items():
+            out[k] = tuple(int(getattr(model, b)[o: o + n].view(torch.int32 if b != "params_bf16" else torch.int16)
+                               .sum(dtype=torch.int64).item()) for b in ("master", "m", "v", "params_bf16"))
+        return out
+
+    kw = dict(step=1, lr=1e-4, b1=0.9, b2=0.95, weight_decay=0.1, no_decay_modules=["embedding.weight"])
+    res = []
+    for overlap in (False, True):
+        model.reset_parameters(0)
+        model.init_optimizer_state()
+        loss = model.train_step(ids, labels, overlap_optimizer=overlap, **kw).item()
+        n_launch = _lib.load().olmax_model_last_step_overlapped_launches()
+        assert (n_launch >= 34 + 32) if overlap else n_launch == 0, n_launch  # 32 layers + norm + embedding, 32 head pieces
+        torch.cuda.synchronize()
+        res.append((loss, checksums()))
+    assert res[0][0] == res[1][0] == loss_ac
+    assert res[0][1] == res[1][1]
 
 
 @pytest.mark.parametrize("name", ["llama3_8B", "olmo2_32B"])

@@ -394,6 +394,36 @@ def test_cross_entropy(T, V, f32, cap):
     assert ((lse.cpu().double() - wlse * mask).abs().max()) < 2e-3
 
 
+@pytest.mark.parametrize("V,f32", [(100352, False), (4096, False), (262144, False), (4104, True)])
+def test_cross_entropy_in_place_equals_out_of_place(V, f32):
+    """dlogits may alias logits (olmax_lmhead_ce always calls it that way).  The label's logit is
+    taken before any wave can store a gradient over the row, so the aliased call must give
+    bit-identical loss, lse and gradient; labels sit in the first and the last 128-bit vector of
+    the row, where a late re-read of the row would meet the earliest and the latest stores.
+    Covers the register-resident kernels (8 and 16 waves per row) and the streaming one."""
+    ops = _ops()
+    say(f"ce in place == out of place V{V} f32{f32}")
+    T = 64
+    g = torch.Generator().manual_seed(7)
+    logits = (torch.randn(T, V, generator=g) * 3)
+    logits = (logits if f32 else logits.to(BF)).cuda()
+    labels = torch.randint(0, V, (T,), generator=g, dtype=torch.int32)
+    labels[0::4] = torch.randint(0, 8, (T // 4,), generator=g, dtype=torch.int32)          # first vector
+    labels[1::4] = V - 1 - torch.randint(0, 8, (T // 4,), generator=g, dtype=torch.int32)  # last vector
+    labels = labels.cuda()
+    for cap in (0.0, 30.0):
+        l0, d0, lse0 = ops.cross_entropy(logits, labels, softcap=cap)
+        z = logits.clone()
+        l1, d1, lse1 = ops.cross_entropy(z, labels, softcap=cap, inplace=True)
+        assert d1.data_ptr() == z.data_ptr()
+        assert l0.item() == l1.item() and torch.equal(lse0, lse1) and torch.equal(d0, d1)
+        # and the loss is the mean of lse - z[label] over the rows
+        zl = logits.float().gather(1, labels.long()[:, None])[:, 0]
+        if cap:
+            zl = cap * torch.tanh(zl / cap)
+        assert abs(l0.item() - (lse0 - zl).mean().item()) < 1e-4
+
+
 def test_cross_entropy_reference_invariants():
     """src/test/nn/functional_test.py:10-18: an appended ignore_index row leaves the mean unchanged."""
     ops = _ops()

@@ -246,12 +246,19 @@ def test_single_block_fwd_bwd(kind, full_qk):
         assert cosine(g, G["layers.0." + n]) >= 0.999, n
 
 
+def _overlapped_launches():
+    from olmax_amd import _lib
+    return _lib.load().olmax_model_last_step_overlapped_launches()
+
+
 def test_overlapped_optimizer_equals_sequential():
     """AdamW launched per layer on a second stream during the backward pass gives the same
-    parameters as loss_and_grads followed by the whole-model AdamW."""
+    parameters as loss_and_grads followed by the whole-model AdamW.  The overlapped branch only
+    exists with full-block recompute; the library's launch counter proves which branch ran."""
     say("overlapped optimizer == sequential")
     from olmax_amd import AdamWConfig, ConstantSchedule, Trainer
     ocfg, hcfg = _cfgs("gemma")
+    hcfg.layer_ac_policy = "nothing_saveable"
     B, S = 2, 128
     P = _params(ocfg)
     outs = []
@@ -265,11 +272,104 @@ def test_overlapped_optimizer_equals_sequential():
             ids = torch.randint(0, 512, (B * S,), generator=gen, dtype=torch.int32).cuda()
             labels = torch.randint(0, 512, (B * S,), generator=gen, dtype=torch.int32).cuda()
             losses.append(tr.process_microbatch(ids, labels).item())
+            # final norm, one group per layer, the embedding
+            assert _overlapped_launches() == (hcfg.num_layers + 2 if overlap else 0)
         torch.cuda.synchronize()
         outs.append((losses, model.master.clone(), model.params_bf16.clone()))
     assert outs[0][0] == pytest.approx(outs[1][0], rel=1e-5)
     assert relerr(outs[1][1], outs[0][1]) < 1e-5
     assert (outs[0][2].float() - outs[1][2].float()).abs().max() <= 1e-2 * outs[0][2].float().abs().max()
+
+
+def _untied_llama(n_layers=4, vocab=4112):
+    """An untied Llama-type model whose LM head (vocab x 256) is larger than one layer (655 872
+    parameters), so that the overlapped step cuts the head's update into a layer-sized first piece,
+    even shares that are not multiples of 8 elements (vocab 4112, 4 layers: 132 268) and a clipped
+    last one.  Head dim 128: every bf16 gradient comes from deterministic kernels."""
+    from olmax_amd import TransformerConfig
+    ocfg = ref.ModelConfig(vocab=vocab, d_model=256, n_layers=n_layers, n_heads=2, n_kv_heads=2, head_dim=128, hidden=512,
+                           eps=1e-6, rope_theta=1e4)
+    hcfg = TransformerConfig(vocab_size=vocab, d_model=256, hidden_size=512, num_layers=n_layers, n_heads=2, head_dim=128,
+                             norm_eps=1e-6, rope_theta=1e4, layer_ac_policy="nothing_saveable")
+    return ocfg, hcfg
+
+
+@pytest.mark.parametrize("n_layers,vocab", [(4, 4112), (3, 8200), (5, 2056)])
+def test_overlapped_step_on_an_untied_model_is_bit_equal_to_the_sequential_step(n_layers, vocab):
+    """The measured path: olmax_model_train_step with a second stream, full-block recompute and an
+    UNTIED model, whose LM-head update is spread in pieces over the layers' recompute windows.
+    AdamW is elementwise and the bf16 gradients are deterministic, so from the same state both
+    orders must leave master, m, v and the bf16 working copy of every bf16-gradient leaf BIT-equal
+    (a skipped, doubled or misaligned range of the head cannot hide); leaves whose gradients are
+    summed by fp32 atomics (embedding, norm weights) agree to rounding noise.  Three consecutive
+    steps (non-zero moments, step counts 1-3), each started from the sequential run's state.
+    (vocab 2056: head smaller than a layer, one piece; 8200 x 3 layers: head of 3.2 layers.)"""
+    say(f"overlapped untied train step, bitwise, layers={n_layers} vocab={vocab}")
+    ocfg, hcfg = _untied_llama(n_layers, vocab)
+    B, S = 2, 128
+    P = _params(ocfg)
+    seq = hcfg.build(batch_size=B, sequence_length=S); seq.load_state_dict(P)
+    ovl = hcfg.build(batch_size=B, sequence_length=S); ovl.load_state_dict(P)
+    for mdl in (seq, ovl):
+        mdl.init_optimizer_state()
+    kw = dict(lr=1e-3, b1=0.9, b2=0.95, weight_decay=0.1, no_decay_modules=["embedding.weight"])
+    for step in range(1, 4):
+        gen = torch.Generator().manual_seed(40 + step)
+        ids = torch.randint(0, vocab, (B * S,), generator=gen, dtype=torch.int32).cuda()
+        labels = torch.randint(0, vocab, (B * S,), generator=gen, dtype=torch.int32).cuda()
+        for name in ("master", "m", "v", "params_bf16"):
+            getattr(ovl, name).copy_(getattr(seq, name))
+        l0 = seq.train_step(ids, labels, step=step, overlap_optimizer=False, **kw).item()
+        assert _overlapped_launches() == 0
+        l1 = ovl.train_step(ids, labels, step=step, overlap_optimizer=True, **kw).item()
+        n_launch = _overlapped_launches()
+        assert n_launch >= n_layers + 2, n_launch  # layers, final norm (+ head pieces), embedding
+        torch.cuda.synchronize()
+        assert l0 == l1
+        assert torch.equal(seq.grad_bf16, ovl.grad_bf16)
+        for leaf in seq.leaves:
+            sl = slice(leaf.offset, leaf.offset + leaf.numel)
+            name = seq.leaf_name(leaf)
+            for buf in ("master", "m", "v", "params_bf16"):
+                a, b = getattr(seq, buf)[sl], getattr(ovl, buf)[sl]
+                if not leaf.grad_f32:
+                    assert torch.equal(a, b), (step, name, buf, (a.float() - b.float()).abs().max().item())
+                else:
+                    assert (a.float() - b.float()).abs().max().item() <= 1e-5 * a.float().abs().max().item() + 1e-12, (step, name, buf)
+        # every element of the head moved (Adam's first steps are ~lr in size wherever g != 0)
+        head = next(l for l in seq.leaves if seq.leaf_name(l) == "lm_head.proj.weight")
+        if step == 1:
+            moved = ovl.master[head.offset: head.offset + head.numel] != P["lm_head.proj.weight"].cuda().reshape(-1)
+            assert moved.float().mean().item() > 0.999
+
+
+def test_overlapped_untied_ten_steps_follow_oracle():
+    """The same untied, checkpointed, overlapped configuration driven through Trainer for 10 steps
+    against the oracle's train_step (bf16 compute): loss curve and final parameters."""
+    say("overlapped untied llama 10 steps vs oracle")
+    from olmax_amd import AdamWConfig, ConstantSchedule, Trainer
+    ocfg, hcfg = _untied_llama(4, 4112)
+    B, S = 2, 128
+    master = ref.init_params(ocfg, seed=2)
+    model = hcfg.build(batch_size=B, sequence_length=S)
+    model.load_state_dict(master)
+    tr = Trainer(model, AdamWConfig(lr=ConstantSchedule(3e-4), b1=0.9, b2=0.95, weight_decay=0.1), overlap_optimizer=True)
+    opt = {"m": {k: torch.zeros_like(v) for k, v in master.items()}, "v": {k: torch.zeros_like(v) for k, v in master.items()}}
+    got, want = [], []
+    for step in range(1, 11):
+        gen = torch.Generator().manual_seed(70 + step)
+        ids = torch.randint(0, 4112, (B, S), generator=gen, dtype=torch.int32)
+        labels = torch.randint(0, 4112, (B, S), generator=gen, dtype=torch.int32)
+        got.append(tr.process_microbatch(ids.cuda().reshape(-1), labels.cuda().reshape(-1)).item())
+        assert _overlapped_launches() > 0
+        want.append(ref.train_step(ocfg, master, opt, ids, labels.long(), step=step, lr=3e-4, b1=0.9, b2=0.95, wd=0.1,
+                                   no_decay=(), compute_bf16=True)[0].item())
+    print("hip   :", [round(x, 4) for x in got]); print("oracle:", [round(x, 4) for x in want], flush=True)
+    for a, b in zip(got, want):
+        assert abs(a - b) < 1e-2 * abs(b)
+    for n, p in model.named_parameters().items():
+        assert relerr(p, master[n]) < 1e-2, n
+    assert torch.equal(model.params_bf16, model.master.to(BF))
 
 
 def test_train_batch_gradient_accumulation_follows_oracle_and_mean_identity():

@@ -312,7 +312,7 @@ def test_rope_tables_fp32_follow_reference_arithmetic():
     assert (cos.double() - c64).abs().max() > 1e-5
 
 
-def _torch_block(kind, P, pre, x, *, H, K, Dh, eps, theta, act, qk):
+def _torch_block(kind, P, pre, x, *, H, K, Dh, eps, theta, act, qk, window=None):
     """One transformer block written from the reference's three forward() bodies
     (src/olmax/nn/transformer/layer.py:86,90 / 108,112 / 175-177,181) and
     MultiheadSelfAttention.forward (src/olmax/nn/attention.py:270-317) with torch's own
@@ -339,8 +339,13 @@ def _torch_block(kind, P, pre, x, *, H, K, Dh, eps, theta, act, qk):
         if qk == "head":
             q, k = norm(q, "attention.q_norm.weight"), norm(k, "attention.k_norm.weight")
         q, k = rope(q), rope(k)
+        if window is None:
+            kw = dict(is_causal=True)
+        else:  # keys i - window .. i (jax.nn.dot_product_attention's local_window_size=(window, 0) under is_causal)
+            i, j = torch.arange(S)[:, None], torch.arange(S)[None, :]
+            kw = dict(attn_mask=(j <= i) & (j >= i - window))
         o = F.scaled_dot_product_attention(q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3),
-                                           is_causal=True, enable_gqa=True).permute(0, 2, 1, 3)
+                                           enable_gqa=True, **kw).permute(0, 2, 1, 3)
         return F.linear(o.reshape(B, S, H * Dh), P[pre + "attention.o_proj.weight"])
 
     def mlp(t):
@@ -386,6 +391,31 @@ def test_block_orderings_against_independent_torch_block(kind, qk):
         other = _torch_block("reordered" if kind == "pre" else "pre", P, "layers.0.", x, H=H, K=K, Dh=6, eps=1e-5,
                              theta=777.0, act=cfg.act, qk=qk)
         assert (ref.block_fwd(cfg, P, 0, x)[0] - other).abs().max() > 1e-3
+
+
+def test_per_layer_theta_and_window_reach_the_right_layer():
+    """cfg.theta(l) / cfg.window(l) inside ref.block_fwd: two Gemma layers with different RoPE
+    bases, the first with a 5-key window, the second global (GemmaTransformerLayer,
+    src/olmax/nn/transformer/layer.py:169-185; per-layer tables as RotaryEmbedding builds them,
+    src/olmax/nn/rope.py:118-145), each against the independent torch block given that layer's own
+    theta and window - and NOT equal to the block built with the other layer's settings."""
+    cfg = ref.ModelConfig(vocab=11, d_model=24, n_layers=2, n_heads=4, n_kv_heads=2, head_dim=6, hidden=40,
+                          layer_type="gemma", act="gelu", qk_norm=True, qk_norm_headwise=True, eps=1e-5, rope_theta=123.0,
+                          rope_theta_layers=[50.0, 9000.0], windows=[4, None])
+    P = _random_block_params(cfg, seed=8)
+    x = torch.randn(2, 13, 24, dtype=D64)
+    settings = [(50.0, 4), (9000.0, None)]
+    for l, (theta, window) in enumerate(settings):
+        kw = dict(H=4, K=2, Dh=6, eps=1e-5, act="gelu", qk="head")
+        want = _torch_block("gemma", P, f"layers.{l}.", x, theta=theta, window=window, **kw)
+        got, _ = ref.block_fwd(cfg, P, l, x)
+        assert torch.allclose(got, want, atol=2e-6), (l, (got - want).abs().max())
+        o_theta, o_window = settings[1 - l]
+        assert (got - _torch_block("gemma", P, f"layers.{l}.", x, theta=o_theta, window=window, **kw)).abs().max() > 1e-3
+        assert (got - _torch_block("gemma", P, f"layers.{l}.", x, theta=theta, window=o_window, **kw)).abs().max() > 1e-3
+    # a window of w shows w + 1 keys: w = 3 differs from w = 4 at 13 tokens
+    assert (_torch_block("gemma", P, "layers.0.", x, theta=50.0, window=3, H=4, K=2, Dh=6, eps=1e-5, act="gelu", qk="head")
+            - ref.block_fwd(cfg, P, 0, x)[0]).abs().max() > 1e-4
 
 
 def test_block_ordering_scale_invariants():
