@@ -164,6 +164,76 @@ def hbm_kernels(T: int, d: int, F: int, heads: int, V: int):
     return out
 
 
+def secondary_config(args):
+    """The other BASELINE workloads at their real widths, as a clearly labelled secondary leg
+    (--config 2 | 4 | 5; never the headline): ms per step and the share of the 2.5 PFLOP/s bf16
+    peak the step's model FLOPs reach, beside the ideal step time.
+      2: one OLMo2-7B block, forward + backward in isolation, activations [2, 4096, 4096];
+      4: Gemma2-27B-like 4-layer slice + embedding + LM head + CE, forward + backward;
+      5: Gemma3-27B-like 6-layer slice, forward + backward + the fused AdamW step."""
+    import torch
+    from olmax_amd import TransformerRecipe
+    from olmax_amd.layer import TransformerBlock
+
+    B, S = 2, 4096
+    T = B * S
+    gen = torch.Generator().manual_seed(0)
+    k = args.config
+    if k == 2:
+        cfg = TransformerRecipe.olmo2_7B_block_bench()
+        blk = TransformerBlock(cfg, batch_size=B, sequence_length=S)
+        g = torch.Generator(device="cuda").manual_seed(0)
+        for w in (blk.wqkv, blk.wo, blk.wgu, blk.wdown):
+            w.normal_(0.0, 0.02, generator=g)
+        x = torch.randn(T, cfg.d_model, device="cuda", generator=g).to(torch.bfloat16)
+        dy = torch.randn(T, cfg.d_model, device="cuda", generator=g).to(torch.bfloat16)
+
+        def step():
+            blk.forward(x)
+            blk.backward(dy)
+        d, H, K, D, F = cfg.d_model, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.hidden_size
+        flops = 3.0 * T * (2 * d * (H + 2 * K) * D + 2 * H * D * d + 6 * d * F + 4 * H * D * (S + 1) / 2)
+        what = ("one OLMo2-7B block forward+backward (configs[1]): d_model 4096, 32x128 heads, SwiGLU 11008, post-norm + "
+                "head-wise QK-norm, theta 5e5, activations [2, 4096, 4096] bf16")
+        params = blk.wqkv.numel() + blk.wo.numel() + blk.wgu.numel() + blk.wdown.numel()
+    else:
+        cfg = TransformerRecipe.gemma2_slice_bench() if k == 4 else TransformerRecipe.gemma3_slice_bench()
+        model = cfg.build(batch_size=B, sequence_length=S, seed=0)
+        ids = torch.randint(0, cfg.vocab_size, (T,), generator=gen, dtype=torch.int32).cuda()
+        labels = torch.randint(0, cfg.vocab_size, (T,), generator=gen, dtype=torch.int32).cuda()
+        count = [0]
+        if k == 4:
+            def step():
+                model.loss_and_grads(ids, labels)
+            what = ("Gemma2-27B-like 4-layer slice forward+backward (configs[3]): d_model 4608, 32/16 heads x 128, GeGLU 36864, "
+                    "pre+post norm, 4096-window / global layers alternating, soft-caps 50 / 30, vocab 256000 tied, seq 4096, mb 2")
+        else:
+            def step():
+                count[0] += 1
+                model.train_step(ids, labels, step=count[0], lr=1e-4, b1=0.9, b2=0.95, weight_decay=0.1,
+                                 no_decay_modules=["embedding.weight"], overlap_optimizer=not args.no_overlap)
+            what = ("Gemma3-27B-like 6-layer slice forward+backward+AdamW (configs[4]): d_model 5376, 32/16 heads x 128, QK-norm, "
+                    "1024-token windows on 5 of 6 layers, theta 1e4 / 1e6, GeGLU 21504, vocab 262144 tied, seq 4096, mb 2")
+        flops = cfg.flops_per_token(S) * T
+        params = model.num_params
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / max(1, args.steps) * 1e3
+    ideal = flops / PEAK_BF16 * 1e3
+    print(json.dumps({
+        "metric": f"SECONDARY LEG (not the headline): ms/step and share of the bf16 peak, BASELINE configs[{k - 1}]",
+        "value": T / ms * 1e3, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (uniform tokens / N(0,1) activations, N(0,0.02) init, resident in HBM)",
+        "mfu_bf16": ideal / ms, "tflop_per_step": flops / 1e12, "ideal_ms_at_2.5_PFLOPs": ideal,
+        "config": {"workload": what, "params": params, "global_batch": B, "seq_len": S}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -175,6 +245,8 @@ def main():
     ap.add_argument("--no-keep-activations-leg", action="store_true", help="skip the extra measurement without recompute")
     ap.add_argument("--no-overlap", action="store_true", help="run AdamW after the backward pass instead of overlapping it on a second stream")
     ap.add_argument("--profiler-ranges", action="store_true", help="emit roctx ranges per layer and phase (for rocprofv3 --marker-trace)")
+    ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5],
+                    help="BASELINE workload (1-based): 3 = the headline Llama-like 7B step (default); 2, 4, 5 = secondary legs")
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline metric)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -188,6 +260,9 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(1)
     L = _lib.load()
+    if args.config != 3:
+        secondary_config(args)
+        return
     if args.profiler_ranges:
         Trainer.set_profiler_ranges(True)
     B, S = 2, 4096

@@ -51,8 +51,10 @@ int32_t olmax_abi_version(void);
  * the two products JAX autodiff derives from it (dx = dy W, dW = dy^T x).
  * C[M,N] = A B^T (+ R).  a_layout/b_layout 0: operand stored with the reduction dimension
  * contiguous (A [M,K], B [N,K]); 1: stored transposed (A [K,M], B [K,N]).
- * R (optional bf16 [M,N]) is added in fp32 before the single rounding of C (residual add of
- * src/olmax/nn/transformer/layer.py:86,90).  out_f32 != 0 writes C as fp32. */
+ * R (optional bf16 [M,N]) is the residual of src/olmax/nn/transformer/layer.py:86,90, `x + linear(..)`
+ * on bf16 arrays: C = bf16(bf16(A B^T) + R), the product rounded to bf16 first as the reference's
+ * linear output is, the sum rounded again (with out_f32 != 0: C = fp32(A B^T) + R, fp32, unrounded).
+ * out_f32 != 0 writes C as fp32. */
 int32_t olmax_gemm_bf16(olmax_stream_t stream, const void* A, const void* B, void* C, const void* R,
                         int32_t M, int32_t N, int32_t K, int64_t lda, int64_t ldb, int64_t ldc,
                         int64_t ldr, int32_t a_layout, int32_t b_layout, int32_t out_f32);
@@ -363,6 +365,10 @@ int32_t olmax_block_bwd(olmax_stream_t stream, const olmax_model_config* cfg, co
 /* Force the MFMA tile variant of olmax_gemm_bf16 (0 = automatic, 128, 256).  While set, the
  * fused GLU / RoPE projections take their unfused paths (same results). */
 void olmax_gemm_set_tile(int tile);
+/* Order in which the MFMA GEMM's workgroups take their tiles: 0 = automatic (per shape and operand
+ * layout), -1 = one contiguous run of tiles per XCD, n > 0 = windows of 8 x 4 tiles per XCD whose 8
+ * windows in flight cover n strips of 8 tile rows (n = 1, 2, 4, 8).  Results do not depend on it. */
+void olmax_gemm_set_order(int order);
 /* Record a HIP-event pair on the launch stream around every MFMA GEMM launch between begin and
  * end (allocates events).  end() waits for them and aggregates per kernel instantiation:
  * key = tile | a_kc<<12 | b_kc<<13 | has_res<<14 | out_f32<<15 | glu_epilogue<<16 |
@@ -371,6 +377,8 @@ void olmax_gemm_set_tile(int tile);
 void olmax_gemm_profile_begin(void);
 int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flops, double* bytes, int64_t* launches,
                                int32_t cap);
+/* The same, aggregated per (key, M, N, K): mnk receives three ints per entry. */
+int32_t olmax_gemm_profile_end_shapes(int32_t* keys, int32_t* mnk, double* ms, int64_t* launches, int32_t cap);
 /* Profiler ranges: the counterpart of the reference's jax.named_scope annotations and
  * ProfilerCallback (src/olmax/train/callbacks/profiler.py:33-50).  on != 0: the whole-model entry
  * points emit roctx ranges ("olmax.layers.<l>.forward" / ".backward", "olmax.lm_head_and_loss")

@@ -52,6 +52,7 @@ struct ProfRec {
   double flops;
   double bytes;  // algorithmic: every operand and the result moved once
   int key;  // tile | a_kc<<12 | b_kc<<13 | has_res<<14 | out_f32<<15
+  int M, N, K;
 };
 std::atomic<bool> g_prof_on{false};  // diagnostic switch, process-wide
 std::vector<ProfRec> g_prof;
@@ -73,7 +74,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
     const bf16* __restrict__ A, const bf16* __restrict__ B, void* __restrict__ Cv,
     const bf16* __restrict__ R, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
     int64_t ldr, int tiles_m, int tiles_n, int c_vec, const float* __restrict__ cos_t,
-    const float* __restrict__ sin_t, int seq_len, int rope_cols) {
+    const float* __restrict__ sin_t, int seq_len, int rope_cols, int order) {
   constexpr int GLU = (EPI == 1 || EPI == 2) ? EPI : 0;
   constexpr bool ROPE = EPI == 3;
   static_assert(EPI == 0 || (BN == 256 && WN == 64 && B_KC && !HAS_RES && !OUT_F32), "fused epilogues: 256-wide NT tiles only");
@@ -96,18 +97,41 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   // ---- XCD-aware tile assignment ----
   const int nwg = gridDim.x;
   int pid = blockIdx.x;
-  {
-    const int per = nwg >> 3;
-    if ((nwg & 7) == 0) pid = (pid & 7) * per + (pid >> 3);
+  int tile_m, tile_n;
+  if (order > 0) {
+    // Windows of 8 x 4 tiles (what the 32 CUs of an XCD hold at a time: 12 operand panels for
+    // 32 tiles in that XCD's L2), dealt to the XCDs so that the 8 windows in flight together
+    // form one block of `order` 8-row strips by 32 / order columns (order 2: 16 x 16 tiles, 32
+    // distinct panels per round for the whole chip; order 4: 32 x 8; order 8: 64 x 4).  Groups of
+    // `order` strips sweep all columns before the next group starts, so B is read once per group
+    // and a group's A panels are re-read from the memory-side cache on every step of the sweep.
+    // The tile grid is padded to whole windows and the launch to whole rounds; workgroups that
+    // fall into the padding leave at once.
+    const int xcd = pid & 7, slot = pid >> 3;
+    const int c = (slot >> 5) * 8 + xcd, w = slot & 31;  // window, tile inside the window
+    const int strips = (tiles_m + 7) >> 3, wpr = (tiles_n + 3) >> 2;  // 8-row strips, windows per strip
+    if (c >= strips * wpr) return;
+    const int full = (strips / order) * order * wpr;      // windows in whole groups of strips
+    int sg, v, S;
+    if (c < full) { sg = c / (order * wpr); v = c % (order * wpr); S = order; }
+    else { sg = strips / order; v = c - full; S = strips % order; }
+    tile_m = ((order * sg + v % S) << 3) + (w & 7);
+    tile_n = ((v / S) << 2) + (w >> 3);
+    if (tile_m >= tiles_m || tile_n >= tiles_n) return;
+  } else {
+    {
+      const int per = nwg >> 3;
+      if ((nwg & 7) == 0) pid = (pid & 7) * per + (pid >> 3);
+    }
+    // column-grouped walk: groups of GM row-tiles, sweep N inside a group
+    constexpr int GM = 8;
+    const int group_sz = GM * tiles_n;
+    const int gid = pid / group_sz;
+    const int first_m = gid * GM;
+    const int gm = min(tiles_m - first_m, GM);
+    tile_m = first_m + (pid % group_sz) % gm;
+    tile_n = (pid % group_sz) / gm;
   }
-  // column-grouped walk: groups of GM row-tiles, sweep N inside a group
-  constexpr int GM = 8;
-  const int group_sz = GM * tiles_n;
-  const int gid = pid / group_sz;
-  const int first_m = gid * GM;
-  const int gm = min(tiles_m - first_m, GM);
-  const int tile_m = first_m + (pid % group_sz) % gm;
-  const int tile_n = (pid % group_sz) / gm;
   const int m0 = tile_m * BM, n0 = tile_n * (GLU ? BN / 2 : BN);  // GLU: first feature of the block
 
   // swizzles (see the bank-geometry note at the top of the file)
@@ -470,8 +494,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
   if (!OUT_F32 && c_vec) {
     // Through LDS (free now), so that C leaves in whole 128-byte lines: each wave parks its
     // WM x 64 tile as bf16 rows of 128 B (16-byte chunks swizzled like the operand tiles), reads
-    // it back 16 B per lane -- 8 lanes per row -- and stores 8 full lines per instruction.  The
-    // residual is added in fp32 before the single rounding, as in the reference.
+    // it back 16 B per lane -- 8 lanes per row -- and stores 8 full lines per instruction.  A
+    // residual joins on the way out, read in the same whole-line pattern: y = bf16(bf16(A B^T) + r),
+    // the two roundings of the reference's `x + linear(...)` on bf16 arrays.
     static_assert(WN == 64, "the staging layout assumes 64-column wave tiles");
     __syncthreads();  // every wave is done reading the operand stages
     unsigned char* ws = smem + wave * (WM * 128);
@@ -481,18 +506,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
       for (int j = 0; j < TN; j++) {
         const int row = i * 16 + l16e;
         const int chunk = j * 2 + (g16e >> 1);
-        float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) v[r] = acc[i][j][r];
-        if (HAS_RES) {
-          Pack4 rr;
-          rr.u = *reinterpret_cast<const u32x2*>(R + (int64_t)(m0 + wm * WM + row) * ldr + n0 + wn * WN + j * 16 + g16e * 4);
-#pragma unroll
-          for (int r = 0; r < 4; r++) v[r] += bf2f(rr.e[r]);
-        }
         Pack4 pk;
 #pragma unroll
-        for (int r = 0; r < 4; r++) pk.e[r] = f2bf(v[r]);
+        for (int r = 0; r < 4; r++) pk.e[r] = f2bf(acc[i][j][r]);
         *reinterpret_cast<u32x2*>(ws + row * 128 + ((chunk ^ kswz(row)) << 4) + ((g16e & 1) << 3)) = pk.u;
       }
     bf16* C = reinterpret_cast<bf16*>(Cv);
@@ -527,6 +543,24 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
       }
       return;
     }
+    if (HAS_RES) {
+      Pack8 rr[WM / 8];
+#pragma unroll
+      for (int t = 0; t < WM / 8; t++) {  // all residual lines requested before the first is needed
+        const int row = t * 8 + (lane_e >> 3), chunk = lane_e & 7;
+        rr[t].u = *reinterpret_cast<const u32x4*>(R + (int64_t)(m0 + wm * WM + row) * ldr + n0 + wn * WN + chunk * 8);
+      }
+#pragma unroll
+      for (int t = 0; t < WM / 8; t++) {
+        const int row = t * 8 + (lane_e >> 3), chunk = lane_e & 7;
+        Pack8 line, o;
+        line.u = *reinterpret_cast<const u32x4*>(ws + row * 128 + ((chunk ^ kswz(row)) << 4));
+#pragma unroll
+        for (int e = 0; e < 8; e++) o.e[e] = f2bf(bf2f(line.e[e]) + bf2f(rr[t].e[e]));
+        *reinterpret_cast<u32x4*>(C + (int64_t)(m0 + wm * WM + row) * ldc + n0 + wn * WN + chunk * 8) = o.u;
+      }
+      return;
+    }
 #pragma unroll
     for (int t = 0; t < WM / 8; t++) {
       const int row = t * 8 + (lane_e >> 3), chunk = lane_e & 7;
@@ -545,7 +579,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
       for (int r = 0; r < 4; r++) {
         const int col = n0 + wn * WN + j * 16 + g16e * 4 + r;
         float v = acc[i][j][r];
-        if (HAS_RES) v += bf2f(R[row * ldr + col]);
+        if (HAS_RES) v = (OUT_F32 ? v : bf2f(f2bf(v))) + bf2f(R[row * ldr + col]);  // bf16 output: round, add, round
         if (OUT_F32)
           reinterpret_cast<float*>(Cv)[row * ldc + col] = v;
         else
@@ -578,12 +612,37 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(
     __syncthreads();
   }
   if (row < M && col < N) {
-    if (R) acc += bf2f(R[(int64_t)row * ldr + col]);
+    if (R) acc = (OUT_F32 ? acc : bf2f(f2bf(acc))) + bf2f(R[(int64_t)row * ldr + col]);
     if (OUT_F32)
       reinterpret_cast<float*>(Cv)[(int64_t)row * ldc + col] = acc;
     else
       reinterpret_cast<bf16*>(Cv)[(int64_t)row * ldc + col] = f2bf(acc);
   }
+}
+
+std::atomic<int> g_order{0};  // diagnostic override of the tile order, process-wide: 0 automatic, -1 run order, > 0 that many strips
+// How many 8-row strips of tiles the 8 XCDs' windows cover together (see the kernel), 0: the
+// run order.  Measured inside the 7B train step (same box, alternating settings, per shape):
+//   forward (both operands k-contiguous), weights that fit the memory-side cache: 1 strip
+//     (all XCDs share the same 8 activation row panels and stream the weights): q|k|v -4.7 %;
+//     a weight matrix beyond the cache (the LM head) wants every row in flight instead;
+//   input gradients (dX = dY W): 2 strips, -2 % at K = 4096, -3.5 % on the LM head, else neutral;
+//   weight gradients (dW = dY^T X): 4 strips, -3 % to -5 % on every shape.
+// Grids that would need padded windows keep the run order (the padding costs more than it gains).
+int tile_order(int tm, int tn, bool a_kc, bool b_kc, int N, int K) {
+  const int o = g_order.load(std::memory_order_relaxed);
+  if (o < 0) return 0;
+  if (o > 0) return o;
+  if (tm % 8 || tn % 4) return 0;
+  const int strips = tm / 8;
+  if (a_kc && b_kc) return (int64_t)N * K * 2 <= (128ll << 20) ? 1 : (strips < 8 ? strips : 8);
+  if (a_kc) return strips < 2 ? strips : 2;
+  return strips < 4 ? strips : 4;
+}
+unsigned order_grid(int order, int tm, int tn) {
+  if (order <= 0) return (unsigned)(tm * tn);
+  const int nwin = ((tm + 7) / 8) * ((tn + 3) / 4);
+  return (unsigned)((nwin + 7) / 8 * 256);
 }
 
 template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool HAS_RES, bool OUT_F32>
@@ -601,15 +660,17 @@ int launch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16
     (void)hipEventCreate(&rec.e1);
     (void)hipEventRecord(rec.e0, s);
   }
-  // vector epilogue: 16-byte stores to C, 8-byte loads from R
-  const int c_vec = aligned16(C) && ldc % 8 == 0 && (!R || ((((uintptr_t)R) & 7) == 0 && ldr % 4 == 0));
-  hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(NT), SMEM, s, A, B, C, R, M, N, K, lda, ldb, ldc,
-                     ldr, tm, tn, c_vec, (const float*)nullptr, (const float*)nullptr, 1, 0);
+  // vector epilogue: 16-byte stores to C, 16-byte loads from R
+  const int c_vec = aligned16(C) && ldc % 8 == 0 && (!R || (aligned16(R) && ldr % 8 == 0));
+  const int order = tile_order(tm, tn, A_KC, B_KC, N, K);
+  hipLaunchKernelGGL(kern, dim3(order_grid(order, tm, tn)), dim3(NT), SMEM, s, A, B, C, R, M, N, K, lda, ldb, ldc,
+                     ldr, tm, tn, c_vec, (const float*)nullptr, (const float*)nullptr, 1, 0, order);
   if (g_prof_on) {
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 2.0 * M * N * K;
     rec.bytes = 2.0 * ((double)M * K + (double)N * K + (double)M * N * (HAS_RES ? 2 : 1) * (OUT_F32 ? 2 : 1));
     rec.key = (BM == 256 ? 256 : 128) | (A_KC << 12) | (B_KC << 13) | (HAS_RES << 14) | (OUT_F32 << 15);
+    rec.M = M; rec.N = N; rec.K = K;
     std::lock_guard<std::mutex> lk(g_prof_mu);
     g_prof.push_back(rec);
   }
@@ -634,13 +695,15 @@ int launch_glu(hipStream_t s, const bf16* A, const bf16* B, bf16* gu, bf16* act,
   // 2: 16-byte stores of whole lines through LDS; 1: 8-byte stores straight from the accumulators
   const int c_vec = (aligned16(act) && ldact % 8 == 0 && (!gu || (aligned16(gu) && ldgu % 8 == 0 && F % 8 == 0))) ? 2
                     : ((((uintptr_t)act) & 7) == 0 && ldact % 4 == 0 && (!gu || ((((uintptr_t)gu) & 7) == 0 && ldgu % 4 == 0 && F % 4 == 0)));
-  hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(512), SMEM, s, A, B, (void*)gu, (const bf16*)act, M, F, K, lda, ldb,
-                     ldgu, ldact, tm, tn, c_vec, (const float*)nullptr, (const float*)nullptr, 1, 0);
+  const int order = tile_order(tm, tn, true, true, 2 * F, K);
+  hipLaunchKernelGGL(kern, dim3(order_grid(order, tm, tn)), dim3(512), SMEM, s, A, B, (void*)gu, (const bf16*)act, M, F, K, lda, ldb,
+                     ldgu, ldact, tm, tn, c_vec, (const float*)nullptr, (const float*)nullptr, 1, 0, order);
   if (g_prof_on) {
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 4.0 * M * F * K;
     rec.bytes = 2.0 * ((double)M * K + 2.0 * F * K + (double)M * F * (gu ? 3 : 1));
     rec.key = 256 | (1 << 12) | (1 << 13) | (1 << 16);
+    rec.M = M; rec.N = 2 * F; rec.K = K;
     std::lock_guard<std::mutex> lk(g_prof_mu);
     g_prof.push_back(rec);
   }
@@ -663,6 +726,7 @@ std::atomic<int> g_force_tile{0};  // diagnostic override, process-wide
 }  // namespace
 
 extern "C" void olmax_gemm_set_tile(int tile) { g_force_tile = tile; }
+extern "C" void olmax_gemm_set_order(int order) { g_order = order; }
 
 // Start recording a HIP-event pair around every MFMA GEMM launch (diagnostic; allocates events).
 extern "C" void olmax_gemm_profile_begin(void) {
@@ -693,6 +757,31 @@ extern "C" int32_t olmax_gemm_profile_end(int32_t* keys, double* ms, double* flo
       n++;
     }
     ms[i] += t; flops[i] += r.flops; bytes[i] += r.bytes; launches[i] += 1;
+    (void)hipEventDestroy(r.e0);
+    (void)hipEventDestroy(r.e1);
+  }
+  g_prof.clear();
+  return n;
+}
+
+// As olmax_gemm_profile_end, aggregated per (key, M, N, K): mnk receives 3 ints per entry.
+extern "C" int32_t olmax_gemm_profile_end_shapes(int32_t* keys, int32_t* mnk, double* ms, int64_t* launches, int32_t cap) {
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  g_prof_on = false;
+  int n = 0;
+  for (auto& r : g_prof) {
+    (void)hipEventSynchronize(r.e1);
+    float t = 0.f;
+    (void)hipEventElapsedTime(&t, r.e0, r.e1);
+    int i = 0;
+    for (; i < n; i++)
+      if (keys[i] == r.key && mnk[3 * i] == r.M && mnk[3 * i + 1] == r.N && mnk[3 * i + 2] == r.K) break;
+    if (i == n) {
+      if (n >= cap) continue;
+      keys[n] = r.key; mnk[3 * n] = r.M; mnk[3 * n + 1] = r.N; mnk[3 * n + 2] = r.K; ms[n] = 0; launches[n] = 0;
+      n++;
+    }
+    ms[i] += t; launches[i] += 1;
     (void)hipEventDestroy(r.e0);
     (void)hipEventDestroy(r.e1);
   }
@@ -826,13 +915,15 @@ extern "C" int32_t olmax_gemm_rope_bf16(hipStream_t stream, const void* X, const
       (void)hipEventCreate(&rec.e1);
       (void)hipEventRecord(rec.e0, stream);
     }
-    hipLaunchKernelGGL(kern, dim3(tm * tn), dim3(512), SMEM, stream, (const bf16*)X, (const bf16*)W, out, (const bf16*)nullptr, M,
-                       N, K, ldx, ldw, ldo, (int64_t)0, tm, tn, 1, cos_t, sin_t, seq_len, rope_heads * 128);
+    const int order = tile_order(tm, tn, true, true, N, K);
+    hipLaunchKernelGGL(kern, dim3(order_grid(order, tm, tn)), dim3(512), SMEM, stream, (const bf16*)X, (const bf16*)W, out, (const bf16*)nullptr, M,
+                       N, K, ldx, ldw, ldo, (int64_t)0, tm, tn, 1, cos_t, sin_t, seq_len, rope_heads * 128, order);
     if (g_prof_on) {
       (void)hipEventRecord(rec.e1, stream);
       rec.flops = 2.0 * M * N * K;
       rec.bytes = 2.0 * ((double)M * K + (double)N * K + (double)M * N);
       rec.key = 256 | (1 << 12) | (1 << 13) | (1 << 17);
+      rec.M = M; rec.N = N; rec.K = K;
       std::lock_guard<std::mutex> lk(g_prof_mu);
       g_prof.push_back(rec);
     }

@@ -197,6 +197,41 @@ class TransformerRecipe:
                                  n_heads=32, n_kv_heads=16, head_dim=128, layer_type="gemma", activation="gelu",
                                  qk_norm_headwise=True)
 
+    # ---- the other measured / parity-tested workloads, at their real widths
+    @staticmethod
+    def olmo2_7B_block_bench() -> TransformerConfig:
+        """One OLMo2-7B block in isolation (ReorderedNormTransformerLayer, layer.py:102-116, with
+        head-wise QK-norm): d 4096, 32 x 128 heads, SwiGLU 11008, eps 1e-6, theta 5e5."""
+        c = TransformerRecipe.olmo2_7B()
+        c.num_layers, c.norm_eps, c.rope_theta, c.vocab_size = 1, 1e-6, 500_000.0, 8
+        return c
+
+    @staticmethod
+    def gemma2_slice_bench(num_layers: int = 4) -> TransformerConfig:
+        """Gemma2-27B-like slice: d 4608, 32 / 16 heads x 128, GeGLU 36864, pre+post norm, layers
+        alternating a 4096-token window and global attention, attention soft-cap 50, final soft-cap
+        30, vocab 256000 tied, full-block recompute."""
+        c = TransformerRecipe.gemma2_like_27B(num_layers)
+        c.norm_eps, c.rope_theta = 1e-6, 10_000.0
+        c.window_size_per_layer = [4096 if l % 2 == 0 else None for l in range(num_layers)]
+        c.attn_logit_softcap, c.final_logit_softcap, c.tie_embeddings = 50.0, 30.0, True
+        c.layer_ac_policy = "nothing_saveable"
+        return c
+
+    @staticmethod
+    def gemma3_slice_bench(num_layers: int = 6) -> TransformerConfig:
+        """Gemma3-27B-like slice (5 local : 1 global): d 5376, 32 / 16 heads x 128, head-wise QK-norm,
+        1024-token windows and theta 1e4 on local layers, theta 1e6 on the global one, GeGLU 21504,
+        vocab 262144 tied, full-block recompute."""
+        c = TransformerRecipe.gemma3_like_27B(num_layers)
+        c.vocab_size, c.norm_eps = 262_144, 1e-6
+        glob = [(l + 1) % 6 == 0 for l in range(num_layers)]
+        c.window_size_per_layer = [None if g else 1024 for g in glob]
+        c.rope_theta_per_layer = [1e6 if g else 1e4 for g in glob]
+        c.tie_embeddings = True
+        c.layer_ac_policy = "nothing_saveable"
+        return c
+
     @staticmethod
     def tiny_llama() -> TransformerConfig:
         """4 layers, d 256, 4x64 heads, hidden 1024, vocab 4096 (CPU-sized plumbing config)."""

@@ -63,8 +63,11 @@ def test_gemm_layouts(M, N, K, al, bl):
     want = af @ bf_.t()
     got = ops.gemm(a.cuda(), b.cuda(), a_layout=al, b_layout=bl)
     assert maxrel(got, want) < 6e-3
+    plain = got
     got = ops.gemm(a.cuda(), b.cuda(), a_layout=al, b_layout=bl, residual=r.cuda(), out_f32=True)
     assert maxrel(got, want + r.double()) < 1e-5
+    got = ops.gemm(a.cuda(), b.cuda(), a_layout=al, b_layout=bl, residual=r.cuda())
+    assert torch.equal(got, (plain.float() + r.cuda().float()).to(BF))  # bf16(bf16(A B^T) + R), every tile size
 
 
 def test_gemm_brute_force_tiny_and_strided():
@@ -105,6 +108,9 @@ def test_gemm_256_tiles_row_strided_operands(M, N, K, al, bl):
     out = torch.zeros(M, N + 24, device="cuda", dtype=BF)
     ops.gemm(av, bv, a_layout=al, b_layout=bl, residual=rv, out=out[:, 16:16 + N])
     assert maxrel(out[:, 16:16 + N], want + rv.double().cpu()) < 6e-3
+    # the residual joins the ROUNDED product, like the reference's `x + linear(...)` on bf16 arrays:
+    # bit-equal to the plain product plus the residual, rounded once more
+    assert torch.equal(out[:, 16:16 + N], (got.float() + rv.float()).to(BF))
     assert not out[:, :16].any() and not out[:, 16 + N:].any()  # nothing written outside the view
 
 
