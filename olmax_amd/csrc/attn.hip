@@ -156,6 +156,14 @@ struct TileDma {
   }
 };
 
+// acc + sum of the two bf16 values in dword w of a packed fragment
+__device__ __forceinline__ float dot2_ones(const bf16x8& v, int w, float acc) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  const bf2 pair = {v[2 * w], v[2 * w + 1]};
+  const bf2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(pair, ones, acc, false);
+}
+
 __device__ __forceinline__ bf16x8 pack_bf16x8(const f32x16& a, int base) {
   bf16x8 r;
 #pragma unroll
@@ -286,19 +294,28 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
           for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
       }
       const float m_use = (m == -INFINITY) ? 0.f : m;
-      float ps = 0.f;
 #pragma unroll
       for (int jt = 0; jt < 2; jt++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const float p = CAP ? fexp2(st[jt][r] - m_use) : fexp2(__builtin_fmaf(st[jt][r], sc2, -m_use));
-          st[jt][r] = p;
-          ps += p;
-        }
-      lsum += ps;
+        for (int r = 0; r < 16; r++)
+          st[jt][r] = CAP ? fexp2(st[jt][r] - m_use) : fexp2(__builtin_fmaf(st[jt][r], sc2, -m_use));
       bf16x8 pb[4];
 #pragma unroll
       for (int u = 0; u < 4; u++) pb[u] = pack_bf16x8(st[u >> 1], (u & 1) * 8);
+      // row sum of the probabilities AS THE P.V PRODUCT SEES THEM (bf16), two per instruction
+      // (v_dot2c_f32_bf16 against a pair of ones, two accumulators): numerator and denominator
+      // of the softmax then carry the same rounding
+      {
+        float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          ps0 = dot2_ones(pb[u], 0, ps0);
+          ps1 = dot2_ones(pb[u], 1, ps1);
+          ps0 = dot2_ones(pb[u], 2, ps0);
+          ps1 = dot2_ones(pb[u], 3, ps1);
+        }
+        lsum += ps0 + ps1;
+      }
 #pragma unroll
       for (int u = 0; u < 4; u++)
 #pragma unroll
@@ -367,7 +384,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     }
   }
   dlt = half_swap_sum(dlt);
-  if (lhi == 0 && qi < S) DELTA[((int64_t)b * H + h) * S + qi] = dlt;
+  // stored NEGATED: the dK/dV kernel starts its dP accumulators from it, so that dP - delta
+  // comes out of the MFMAs and costs that kernel no subtraction
+  if (lhi == 0 && qi < S) DELTA[((int64_t)b * H + h) * S + qi] = -dlt;
   const float lse2 = LSE[((int64_t)b * H + h) * S + qic] * LOG2E;
   const int j_lo = window >= 0 ? max(0, i0 - window) : 0;
   const int t_lo = j_lo >> 6;
@@ -574,19 +593,23 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
       // window edge or the end of the sequence
       const bool need_mask = (ib < jw0 + 31) || (ib + QT > S) || (window >= 0 && ib + QT - 1 > jw0 + window);
       f32x16 sa, dpa;
+      // accumulator rows are queries i = ib + 8*(r/4) + 4*lhi + r%4; column = key kj.
+      // dP starts from -delta of its query (what DELTA holds): the products then give dP - delta
 #pragma unroll
-      for (int r = 0; r < 16; r++) { sa[r] = 0.f; dpa[r] = 0.f; }
+      for (int g = 0; g < 4; g++) {
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(sdel + g * 8 + lhi * 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++) { sa[g * 4 + e] = 0.f; dpa[g * 4 + e] = d4[e]; }
+      }
 #pragma unroll
       for (int s = 0; s < 8; s++) {
         sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(sq, 0, s), kf[s], sa, 0, 0, 0);
         dpa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(so, 0, s), fa.load_kc(svt, wave * 32, s), dpa, 0, 0, 0);
       }
-      // accumulator rows are queries i = ib + 8*(r/4) + 4*lhi + r%4; column = key kj
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         const int il = g * 8 + lhi * 4;
         const f32x4 l4 = *reinterpret_cast<const f32x4*>(slse + il);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(sdel + il);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = g * 4 + e;
@@ -604,7 +627,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
             p = ok ? p : 0.f;
           }
           sa[r] = p;
-          dpa[r] = p * (dpa[r] - d4[e]) * chain;
+          dpa[r] = p * dpa[r] * chain;
         }
       }
       bf16x8 pb[2], dsb[2];
