@@ -10,6 +10,7 @@
 //                 src/olmax/train/trainer.py:745-752; the bf16 copy replaces the per-step
 //                 cast_tree(params, bf16) of src/olmax/train/trainer.py:728
 #include "common.h"
+#include <atomic>
 
 namespace {
 
@@ -197,6 +198,16 @@ __global__ __launch_bounds__(256) void embed_bwd_kernel(const int32_t* __restric
 // bc1 = 1 - b1^t, bc2 = 1 - b2^t (computed on the host in double), or, with hyper_dev, lr and the
 // two bias corrections read from device memory (a host whose schedule and step count live on
 // the device, like optax's injected hyper-parameters inside a jitted step).
+// p - lr (m_hat / (sqrt(v_hat) + eps) + wd p) with the hardware square root and reciprocal (1 ulp
+// each) instead of the correctly rounded library forms: those expand to ~22 vector instructions
+// per element, and when this kernel shares a CU with a GEMM every vector instruction it issues
+// takes an issue slot from the GEMM's MFMAs.  The update moves by a few 1e-7 of its own size
+// (lr-sized), far below one ulp of p.
+__device__ __forceinline__ float adamw_new_p(float p, float mh, float vh, float lr, float eps, float wd) {
+  const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_sqrtf(vh) + eps);
+  return __builtin_fmaf(-lr, __builtin_fmaf(mh, r, wd * p), p);
+}
+
 template <bool G_BF16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(16))) void adamw_kernel(
     float* __restrict__ p, const void* __restrict__ gv, float* __restrict__ m, float* __restrict__ v,
@@ -238,9 +249,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(16))) void adam
       const float ge = g[e] * gscale;
       mv[e] = b1 * mv[e] + omb1 * ge;
       vv[e] = b2 * vv[e] + omb2 * ge * ge;
-      const float mh = mv[e] * ibc1;
-      const float vh = vv[e] * ibc2;
-      pv[e] = pv[e] - lr * (mh / (sqrtf(vh) + eps) + wd * pv[e]);
+      pv[e] = adamw_new_p(pv[e], mv[e] * ibc1, vv[e] * ibc2, lr, eps, wd);
       sh.e[e] = f2bf(pv[e]);
     }
     __builtin_nontemporal_store(pv, reinterpret_cast<f32x4*>(p) + i);
@@ -256,9 +265,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(16))) void adam
     // change any element's result
     const float mm = b1 * m[i] + omb1 * ge;
     const float vv = b2 * v[i] + omb2 * ge * ge;
-    const float mh = mm * ibc1;
-    const float vh = vv * ibc2;
-    const float pp = p[i] - lr * (mh / (sqrtf(vh) + eps) + wd * p[i]);
+    const float pp = adamw_new_p(p[i], mm * ibc1, vv * ibc2, lr, eps, wd);
     m[i] = mm;
     v[i] = vv;
     p[i] = pp;
