@@ -173,6 +173,15 @@ int32_t olmax_cross_entropy(olmax_stream_t stream, const void* logits, void* dlo
                             const int32_t* labels, float* loss, float* lse_out, void* workspace,
                             int64_t workspace_bytes, int64_t T, int32_t V, int64_t ld, int64_t ldd,
                             int32_t logits_f32, int32_t ignore_index, float softcap, float dloss);
+/* The same with the reference's other reductions (src/olmax/nn/functional.py:84-91): reduction 0
+ * "mean", 1 "sum", 2 "none".  With "none" `loss` is the [T] array of row losses (0 for ignored and
+ * out-of-range labels) and the cotangent of row t is dloss * dloss_rows[t] (dloss_rows: device
+ * fp32 [T], NULL = ones). */
+int32_t olmax_cross_entropy_reduce(olmax_stream_t stream, const void* logits, void* dlogits,
+                                   const int32_t* labels, float* loss, float* lse_out,
+                                   const float* dloss_rows, void* workspace, int64_t workspace_bytes,
+                                   int64_t T, int32_t V, int64_t ld, int64_t ldd, int32_t logits_f32,
+                                   int32_t ignore_index, float softcap, float dloss, int32_t reduction);
 
 /* ---- LM head + cross entropy, forward and backward in one call (three GEMMs around a row kernel;
  * the bf16 logits [T, V] are materialised once in the workspace and overwritten by their gradient,

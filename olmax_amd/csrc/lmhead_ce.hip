@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
     const T* __restrict__ logits, T* __restrict__ dlogits, const int32_t* __restrict__ labels,
     float* __restrict__ row_loss, float* __restrict__ lse_out, const int32_t* __restrict__ n_counted,
     int64_t rows, int V, int64_t ld, int64_t ldd, int32_t ignore_index, float cap, float dloss,
-    int vec_ok) {
+    int vec_ok, const float* __restrict__ drow, int mean) {
   constexpr int VEC = Io<T>::VEC;
   __shared__ float red[4];
   __shared__ float label_logit;
@@ -128,7 +128,8 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
   if (!dlogits) return;
   // ---- pass 2: gradient, in place allowed ----
   T* dr = dlogits + row * ldd;
-  const float scale = (counted && inrange) ? dloss / (float)(*n_counted) : 0.f;
+  // d(reduced loss) / d(row loss): 1/n for "mean", 1 for "sum", the row's own cotangent for "none"
+  const float scale = (counted && inrange) ? dloss * (drow ? drow[row] : 1.f) / (mean ? (float)(*n_counted) : 1.f) : 0.f;
   for (int i = threadIdx.x; i < nvec; i += 256) {
     float f[VEC];
     Io<T>::load(zr + i * VEC, f);
@@ -167,7 +168,8 @@ template <bool CAP, int THREADS, int MAXV>
 __global__ __launch_bounds__(THREADS) void ce_row_regs_kernel(
     const bf16* __restrict__ logits, bf16* __restrict__ dlogits, const int32_t* __restrict__ labels,
     float* __restrict__ row_loss, float* __restrict__ lse_out, const int32_t* __restrict__ n_counted,
-    int V, int64_t ld, int64_t ldd, int32_t ignore_index, float cap, float dloss) {
+    int V, int64_t ld, int64_t ldd, int32_t ignore_index, float cap, float dloss,
+    const float* __restrict__ drow, int mean) {
   constexpr int NW = THREADS / 64;
   __shared__ float red[NW];
   __shared__ float label_logit;
@@ -221,7 +223,8 @@ __global__ __launch_bounds__(THREADS) void ce_row_regs_kernel(
   }
   if (!dlogits) return;
   bf16* dr = dlogits + row * ldd;
-  const float scale = (counted && inrange) ? dloss / (float)(*n_counted) : 0.f;
+  // d(reduced loss) / d(row loss): 1/n for "mean", 1 for "sum", the row's own cotangent for "none"
+  const float scale = (counted && inrange) ? dloss * (drow ? drow[row] : 1.f) / (mean ? (float)(*n_counted) : 1.f) : 0.f;
 #pragma unroll
   for (int i = 0; i < MAXV; i++) {
     const int idx = i * THREADS + threadIdx.x;
@@ -244,15 +247,15 @@ __global__ __launch_bounds__(THREADS) void ce_row_regs_kernel(
   }
 }
 
-// loss = sum(row_loss) / n_counted   (single block; deterministic order)
+// loss = sum(row_loss) / n_counted, or the plain sum (single block; deterministic order)
 __global__ __launch_bounds__(256) void ce_finalize_kernel(const float* __restrict__ row_loss, int64_t T,
                                                           const int32_t* __restrict__ n_counted,
-                                                          float* __restrict__ loss) {
+                                                          float* __restrict__ loss, int mean) {
   __shared__ float red[4];
   float s = 0.f;
   for (int64_t i = threadIdx.x; i < T; i += 256) s += row_loss[i];
   s = block_sum<4>(s, red);
-  if (threadIdx.x == 0) *loss = s / (float)(*n_counted);
+  if (threadIdx.x == 0) *loss = mean ? s / (float)(*n_counted) : s;
 }
 
 }  // namespace
@@ -260,20 +263,26 @@ __global__ __launch_bounds__(256) void ce_finalize_kernel(const float* __restric
 // Workspace: T floats (row losses) + 16 bytes (counted-row count), 16-byte aligned.
 extern "C" int64_t olmax_cross_entropy_workspace_bytes(int64_t T) { return ((T * 4 + 15) / 16) * 16 + 16; }
 
-// logits [T, V] (bf16 when logits_f32 == 0, else fp32) -> *loss (fp32 scalar, device);
-// dlogits (same dtype, may alias logits, may be NULL) <- d loss / d logits * dloss;
-// lse_out (optional, [T]) <- log-normaliser * (label != ignore_index)  (the reference's
-// fused_cross_entropy_loss second output, src/olmax/nn/functional.py:94-121).
-extern "C" int32_t olmax_cross_entropy(hipStream_t stream, const void* logits, void* dlogits,
-                                       const int32_t* labels, float* loss, float* lse_out,
-                                       void* workspace, int64_t workspace_bytes, int64_t T, int32_t V,
-                                       int64_t ld, int64_t ldd, int32_t logits_f32,
-                                       int32_t ignore_index, float softcap, float dloss) {
+// logits [T, V] (bf16 when logits_f32 == 0, else fp32) -> loss (device fp32: a scalar, or [T] row
+// losses for reduction "none"); dlogits (same dtype, may alias logits, may be NULL) <-
+// d loss / d logits times the incoming cotangent (the scalar dloss; for "none" also the per-row
+// device array dloss_rows when given); lse_out (optional, [T]) <- log-normaliser *
+// (label != ignore_index)  (the reference's fused_cross_entropy_loss second output,
+// src/olmax/nn/functional.py:94-121).  reduction: 0 "mean", 1 "sum", 2 "none" (functional.py:84-91).
+extern "C" int32_t olmax_cross_entropy_reduce(hipStream_t stream, const void* logits, void* dlogits,
+                                              const int32_t* labels, float* loss, float* lse_out,
+                                              const float* dloss_rows, void* workspace, int64_t workspace_bytes,
+                                              int64_t T, int32_t V, int64_t ld, int64_t ldd, int32_t logits_f32,
+                                              int32_t ignore_index, float softcap, float dloss, int32_t reduction) {
   OLMAX_CHECK(logits && labels && loss && workspace, OLMAX_ERR_ARG, "olmax_cross_entropy: null pointer");
   OLMAX_CHECK(T > 0 && V > 0 && ld >= V && (!dlogits || ldd >= V), OLMAX_ERR_SHAPE, "olmax_cross_entropy: bad shape T=%ld V=%d", (long)T, V);
+  OLMAX_CHECK(reduction >= 0 && reduction <= 2, OLMAX_ERR_ARG, "olmax_cross_entropy: reduction must be 0 (mean), 1 (sum) or 2 (none)");
+  OLMAX_CHECK(!dloss_rows || reduction == 2, OLMAX_ERR_ARG, "olmax_cross_entropy: a per-row cotangent only goes with reduction none");
   OLMAX_CHECK(workspace_bytes >= olmax_cross_entropy_workspace_bytes(T) && aligned16(workspace), OLMAX_ERR_WORKSPACE, "olmax_cross_entropy: workspace too small or misaligned");
-  float* row_loss = (float*)workspace;
+  // "none": the row kernels write the row losses straight into the caller's array
+  float* row_loss = reduction == 2 ? loss : (float*)workspace;
   int32_t* n_counted = (int32_t*)((char*)workspace + ((T * 4 + 15) / 16) * 16);
+  const int mean = reduction == 0;
   hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(256), 0, stream, labels, T, ignore_index, n_counted);
   const int vecw = logits_f32 ? 4 : 8;
   const int vec_ok = aligned16(logits) && (!dlogits || aligned16(dlogits)) && ld % vecw == 0 && (!dlogits || ldd % vecw == 0);
@@ -282,10 +291,10 @@ extern "C" int32_t olmax_cross_entropy(hipStream_t stream, const void* logits, v
 #define CE_GO(TY, CAPV)                                                                          \
   hipLaunchKernelGGL((ce_row_kernel<TY, CAPV>), grid, dim3(256), 0, stream, (const TY*)logits,   \
                      (TY*)dlogits, labels, row_loss, lse_out, n_counted, T, V, ld, ldd,          \
-                     ignore_index, softcap, dloss, vec_ok)
+                     ignore_index, softcap, dloss, vec_ok, dloss_rows, mean)
 #define CE_REGS(CAPV, TH, MV)                                                                              \
   hipLaunchKernelGGL((ce_row_regs_kernel<CAPV, TH, MV>), grid, dim3(TH), 0, stream, (const bf16*)logits,   \
-                     (bf16*)dlogits, labels, row_loss, lse_out, n_counted, V, ld, ldd, ignore_index, softcap, dloss)
+                     (bf16*)dlogits, labels, row_loss, lse_out, n_counted, V, ld, ldd, ignore_index, softcap, dloss, dloss_rows, mean)
   const bool regs_ok = !logits_f32 && vec_ok && V % 8 == 0;
   if (logits_f32) {
     if (cap) CE_GO(float, true); else CE_GO(float, false);
@@ -298,9 +307,19 @@ extern "C" int32_t olmax_cross_entropy(hipStream_t stream, const void* logits, v
   }
 #undef CE_GO
 #undef CE_REGS
-  hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(256), 0, stream, row_loss, T, n_counted, loss);
+  if (reduction != 2) hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(256), 0, stream, row_loss, T, n_counted, loss, mean);
   OLMAX_LAUNCH_CHECK();
   return OLMAX_OK;
+}
+
+// reduction "mean": what the benchmark's loss_fun and the fused LM head use
+extern "C" int32_t olmax_cross_entropy(hipStream_t stream, const void* logits, void* dlogits,
+                                       const int32_t* labels, float* loss, float* lse_out,
+                                       void* workspace, int64_t workspace_bytes, int64_t T, int32_t V,
+                                       int64_t ld, int64_t ldd, int32_t logits_f32,
+                                       int32_t ignore_index, float softcap, float dloss) {
+  return olmax_cross_entropy_reduce(stream, logits, dlogits, labels, loss, lse_out, nullptr, workspace, workspace_bytes, T, V, ld,
+                                    ldd, logits_f32, ignore_index, softcap, dloss, 0);
 }
 
 // Workspace for the fused LM head: bf16 logits [T, V] + the CE workspace.

@@ -102,6 +102,112 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxLmHeadCe, LmHeadCe,
                               ffi::Ffi::Bind().Ctx<Stream>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>()
                                   .Attr<float>("softcap"));
 
+// ---- RoPE with the optional head-wise QK-norm (RotaryPositionalEmbedding.forward, src/olmax/nn/rope.py:68-80,
+// applied at src/olmax/nn/attention.py:298-300 after the norm of :293-296): x [B,S,H,D], cos/sin [S, D/2] fp32,
+// w [D] (read only when use_norm != 0).
+static ffi::Error QkRopeFwd(hipStream_t st, Buf x, Buf w, Buf cos, Buf sin, Out y, int32_t use_norm, float eps) {
+  auto d = x.dimensions();
+  if (d.size() != 4) return ffi::Error::InvalidArgument("olmax_qk_rope_fwd: x must be [B,S,H,D]");
+  const int64_t tokens = d[0] * d[1];
+  const int32_t Sq = (int32_t)d[1], H = (int32_t)d[2], D = (int32_t)d[3];
+  if (cos.dimensions().size() != 2 || cos.dimensions()[0] < Sq || cos.dimensions()[1] * 2 != D)
+    return ffi::Error::InvalidArgument("olmax_qk_rope_fwd: cos/sin must be [>= S, D/2]");
+  return Status(olmax_qk_rope_fwd(S(st), x.untyped_data(), y->untyped_data(), use_norm ? w.untyped_data() : nullptr,
+                                  (const float*)cos.untyped_data(), (const float*)sin.untyped_data(), tokens, H, D, Sq,
+                                  (int64_t)H * D, (int64_t)H * D, eps));
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxQkRopeFwd, QkRopeFwd,
+                              ffi::Ffi::Bind().Ctx<Stream>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Ret<Buf>()
+                                  .Attr<int32_t>("use_norm").Attr<float>("eps"));
+
+// dw (fp32 [D]) is accumulated into by the kernel: zeroed here first (only with use_norm)
+static ffi::Error QkRopeBwd(hipStream_t st, Buf dy, Buf x, Buf w, Buf cos, Buf sin, Out dx, Out dw, int32_t use_norm,
+                            float eps) {
+  auto d = x.dimensions();
+  if (d.size() != 4) return ffi::Error::InvalidArgument("olmax_qk_rope_bwd: x must be [B,S,H,D]");
+  const int64_t tokens = d[0] * d[1];
+  const int32_t Sq = (int32_t)d[1], H = (int32_t)d[2], D = (int32_t)d[3];
+  const int64_t ld = (int64_t)H * D;
+  if (int32_t rc = olmax_fill_zero(S(st), dw->untyped_data(), (int64_t)dw->size_bytes())) return Status(rc);
+  return Status(olmax_qk_rope_bwd(S(st), dy.untyped_data(), dx->untyped_data(), use_norm ? x.untyped_data() : nullptr,
+                                  use_norm ? w.untyped_data() : nullptr, use_norm ? (float*)dw->untyped_data() : nullptr,
+                                  (const float*)cos.untyped_data(), (const float*)sin.untyped_data(), tokens, H, D, Sq, ld, ld,
+                                  ld, eps));
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxQkRopeBwd, QkRopeBwd,
+                              ffi::Ffi::Bind().Ctx<Stream>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Ret<Buf>()
+                                  .Ret<Buf>().Attr<int32_t>("use_norm").Attr<float>("eps"));
+
+// ---- gated MLP (GatedMLP.forward, src/olmax/nn/mlp.py:69-73): the gate|up projection with the activation in the
+// GEMM epilogue (x [..., K], w = [Wgate; Wup] [2F, K] -> act [..., F] and gate|up [..., 2F] for the backward),
+// and the elementwise backward of act(gate) * up.  act: 0 silu, 1 tanh-gelu.
+static ffi::Error GemmGlu(hipStream_t st, Buf x, Buf w, Out act_out, Out gu_out, int32_t act) {
+  const int32_t K = Last(x), F2 = (int32_t)Rows(w);
+  if (Last(w) != K || (F2 & 1)) return ffi::Error::InvalidArgument("olmax_gemm_glu: w must be [2F, K] with K = x's last dimension");
+  return Status(olmax_gemm_glu_bf16(S(st), x.untyped_data(), w.untyped_data(), gu_out->untyped_data(), act_out->untyped_data(),
+                                    (int32_t)Rows(x), F2 / 2, K, K, K, F2, F2 / 2, act));
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxGemmGlu, GemmGlu,
+                              ffi::Ffi::Bind().Ctx<Stream>().Arg<Buf>().Arg<Buf>().Ret<Buf>().Ret<Buf>().Attr<int32_t>("act"));
+
+// gu [..., 2F] (gate | up), dh [..., F] -> dgu [..., 2F] (dgate | dup)
+static ffi::Error GluBwd(hipStream_t st, Buf gu, Buf dh, Out dgu, int32_t act) {
+  const int32_t F = Last(dh);
+  if (Last(gu) != 2 * F) return ffi::Error::InvalidArgument("olmax_glu_bwd: gu must be [..., 2F] for dh [..., F]");
+  const char* g = (const char*)gu.untyped_data();
+  char* dg = (char*)dgu->untyped_data();
+  return Status(olmax_glu_bwd(S(st), g, g + (int64_t)F * 2, dh.untyped_data(), dg, dg + (int64_t)F * 2, Rows(dh), F, 2 * (int64_t)F,
+                              2 * (int64_t)F, F, 2 * (int64_t)F, 2 * (int64_t)F, act));
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxGluBwd, GluBwd,
+                              ffi::Ffi::Bind().Ctx<Stream>().Arg<Buf>().Arg<Buf>().Ret<Buf>().Attr<int32_t>("act"));
+
+// ---- embedding (Embedding.forward, src/olmax/nn/embedding.py:30-32) and its transpose (dW fp32, zeroed here)
+static ffi::Error EmbedFwd(hipStream_t st, Buf ids, Buf w, Out out) {
+  if (w.dimensions().size() != 2) return ffi::Error::InvalidArgument("olmax_embed_fwd: weight must be [V, d]");
+  return Status(olmax_embed_fwd(S(st), (const int32_t*)ids.untyped_data(), w.untyped_data(), out->untyped_data(),
+                                (int64_t)ids.element_count(), (int32_t)w.dimensions()[1], (int32_t)w.dimensions()[0]));
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxEmbedFwd, EmbedFwd, ffi::Ffi::Bind().Ctx<Stream>().Arg<Buf>().Arg<Buf>().Ret<Buf>());
+
+static ffi::Error EmbedBwd(hipStream_t st, Buf ids, Buf dh, Out dw) {
+  if (dw->dimensions().size() != 2) return ffi::Error::InvalidArgument("olmax_embed_bwd: dW must be [V, d]");
+  if (int32_t rc = olmax_fill_zero(S(st), dw->untyped_data(), (int64_t)dw->size_bytes())) return Status(rc);
+  return Status(olmax_embed_bwd(S(st), (const int32_t*)ids.untyped_data(), dh.untyped_data(), (float*)dw->untyped_data(),
+                                (int64_t)ids.element_count(), (int32_t)dw->dimensions()[1], (int32_t)dw->dimensions()[0]));
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxEmbedBwd, EmbedBwd, ffi::Ffi::Bind().Ctx<Stream>().Arg<Buf>().Arg<Buf>().Ret<Buf>());
+
+// ---- cross entropy on given logits (cross_entropy_loss / fused_cross_entropy_loss, src/olmax/nn/functional.py:70-121):
+// forward -> loss (scalar, or [T] for reduction "none") and the log-normaliser * (label != ignore); backward ->
+// dlogits from per-row cotangents (the wrapper folds 1/n of "mean" into them on the device).
+static ffi::Error CrossEntropyFwd(hipStream_t st, Buf logits, Buf labels, Out loss, Out lse, Out ws, int32_t reduction,
+                                  int32_t ignore_index, float softcap) {
+  const int64_t T = Rows(logits);
+  const int32_t V = Last(logits);
+  return Status(olmax_cross_entropy_reduce(S(st), logits.untyped_data(), nullptr, (const int32_t*)labels.untyped_data(),
+                                           (float*)loss->untyped_data(), (float*)lse->untyped_data(), nullptr, ws->untyped_data(),
+                                           (int64_t)ws->size_bytes(), T, V, V, V, logits.element_type() == ffi::DataType::F32,
+                                           ignore_index, softcap, 1.f, reduction));
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxCrossEntropyFwd, CrossEntropyFwd,
+                              ffi::Ffi::Bind().Ctx<Stream>().Arg<Buf>().Arg<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>()
+                                  .Attr<int32_t>("reduction").Attr<int32_t>("ignore_index").Attr<float>("softcap"));
+
+static ffi::Error CrossEntropyBwd(hipStream_t st, Buf logits, Buf labels, Buf row_cotangent, Out dlogits, Out row_loss, Out ws,
+                                  int32_t ignore_index, float softcap) {
+  const int64_t T = Rows(logits);
+  const int32_t V = Last(logits);
+  if ((int64_t)row_cotangent.element_count() != T) return ffi::Error::InvalidArgument("olmax_cross_entropy_bwd: one cotangent per row");
+  return Status(olmax_cross_entropy_reduce(S(st), logits.untyped_data(), dlogits->untyped_data(), (const int32_t*)labels.untyped_data(),
+                                           (float*)row_loss->untyped_data(), nullptr, (const float*)row_cotangent.untyped_data(),
+                                           ws->untyped_data(), (int64_t)ws->size_bytes(), T, V, V, V,
+                                           logits.element_type() == ffi::DataType::F32, ignore_index, softcap, 1.f, 2));
+}
+XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxCrossEntropyBwd, CrossEntropyBwd,
+                              ffi::Ffi::Bind().Ctx<Stream>().Arg<Buf>().Arg<Buf>().Arg<Buf>().Ret<Buf>().Ret<Buf>().Ret<Buf>()
+                                  .Attr<int32_t>("ignore_index").Attr<float>("softcap"));
+
 // ---- AdamW on one leaf (optax.adamw as built at src/olmax/optim/config.py:136-156).  p, m, v are
 // updated in place: the wrapper aliases results 0-2 to arguments 0, 2, 3 (donated buffers).
 // hyper: fp32 [3] = {lr, 1 - b1^t, 1 - b2^t}, computed on the device by the caller from optax's
@@ -145,6 +251,31 @@ static ffi::Error TrainStep(hipStream_t st, Buf master, Buf m, Buf v, Buf params
   c.eps = eps; c.attn_softcap = attn_softcap; c.final_softcap = final_softcap;
   if ((int)windows.size() != c.n_layers || (int)table_index.size() != c.n_layers)
     return ffi::Error::InvalidArgument("olmax_train_step: windows / table_index need one entry per layer");
+  // every attribute and buffer size is checked against what the library will read before anything is launched
+  const int64_t n_params = olmax_model_num_params(&c);
+  if (n_params < 0) return ffi::Error::InvalidArgument(olmax_last_error_string());
+  const int32_t n_leaf = olmax_model_layout(&c, nullptr, 0);
+  if (leaf_decay.size() != 0 && (int64_t)leaf_decay.size() != n_leaf)
+    return ffi::Error::InvalidArgument("olmax_train_step: leaf_decay must be empty or hold one entry per leaf of olmax_model_layout");
+  if (cos.dimensions().size() != 3 || sin.dimensions().size() != 3 || cos.dimensions()[1] != c.seq_len ||
+      cos.dimensions()[2] * 2 != c.head_dim || sin.dimensions()[0] != cos.dimensions()[0] ||
+      sin.dimensions()[1] != cos.dimensions()[1] || sin.dimensions()[2] != cos.dimensions()[2])
+    return ffi::Error::InvalidArgument("olmax_train_step: cos / sin must be [n_tables, seq_len, head_dim / 2]");
+  for (int l = 0; l < c.n_layers; l++)
+    if (table_index[l] < 0 || table_index[l] >= cos.dimensions()[0])
+      return ffi::Error::InvalidArgument("olmax_train_step: table_index entry outside the cos / sin tables");
+  if ((int64_t)master.element_count() != n_params || (int64_t)m.element_count() != n_params ||
+      (int64_t)v.element_count() != n_params || (int64_t)params.element_count() != n_params ||
+      (int64_t)grad_bf16->element_count() != n_params)
+    return ffi::Error::InvalidArgument("olmax_train_step: master, m, v, params and grad_bf16 must hold olmax_model_num_params elements");
+  if ((int64_t)grad_f32->element_count() != olmax_model_grad_f32_elems(&c))
+    return ffi::Error::InvalidArgument("olmax_train_step: grad_f32 must hold olmax_model_grad_f32_elems elements");
+  if ((int64_t)ws->size_bytes() < olmax_model_workspace_bytes(&c))
+    return ffi::Error::InvalidArgument("olmax_train_step: workspace smaller than olmax_model_workspace_bytes");
+  const int64_t T = (int64_t)c.batch * c.seq_len;
+  if ((int64_t)ids.element_count() != T || (int64_t)labels.element_count() != T || hyper.element_count() != 3 ||
+      norm->element_count() != 2)
+    return ffi::Error::InvalidArgument("olmax_train_step: ids / labels need batch * seq_len entries, hyper 3, norm 2");
   const int64_t table = cos.dimensions()[1] * cos.dimensions()[2];
   std::vector<const float*> cp(c.n_layers), sp(c.n_layers);
   for (int l = 0; l < c.n_layers; l++) {

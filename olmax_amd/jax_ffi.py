@@ -7,6 +7,13 @@ What a maintainer of the reference adds to run its Equinox modules and trainer o
                          ``implementation="hip"`` literal;
 * ``hip_rms_norm``, ``hip_linear``, ``hip_lm_head_cross_entropy`` for the pure functions of
                          src/olmax/nn/functional.py:21,51,70 (+ ``LMHead.forward``, lm_head.py:59-61);
+* ``hip_cross_entropy_loss`` / ``hip_fused_cross_entropy_loss`` for src/olmax/nn/functional.py:70-121 on given
+                         logits (all three reductions; the fused one also returns the log-normaliser);
+* ``hip_rope``           for ``RotaryPositionalEmbedding.forward`` (src/olmax/nn/rope.py:68-80), optionally with the
+                         head-wise QK-norm of src/olmax/nn/attention.py:293-296 folded in;
+* ``hip_gated_mlp_in``   for the gate / up half of ``GatedMLP.forward`` (src/olmax/nn/mlp.py:69-73): one GEMM with the
+                         activation in its epilogue;
+* ``hip_embedding``      for ``Embedding.forward`` (src/olmax/nn/embedding.py:30-32);
 * ``hip_adamw``          an ``optax.GradientTransformation`` for ``optim.update`` at
                          src/olmax/train/trainer.py:745;
 * ``HipTrainStep``       ``process_microbatch`` (src/olmax/train/trainer.py:759-777) as ONE custom call on
@@ -32,7 +39,10 @@ from . import _lib
 FFI_LIB = Path(__file__).resolve().parent / "libolmax_ffi.so"
 _TARGETS = {"olmax_attn_fwd": "OlmaxAttnFwd", "olmax_attn_bwd": "OlmaxAttnBwd", "olmax_rmsnorm_fwd": "OlmaxRmsNormFwd",
             "olmax_rmsnorm_bwd": "OlmaxRmsNormBwd", "olmax_gemm": "OlmaxGemm", "olmax_lmhead_ce": "OlmaxLmHeadCe",
-            "olmax_adamw": "OlmaxAdamW", "olmax_train_step": "OlmaxTrainStep"}
+            "olmax_adamw": "OlmaxAdamW", "olmax_train_step": "OlmaxTrainStep",
+            "olmax_qk_rope_fwd": "OlmaxQkRopeFwd", "olmax_qk_rope_bwd": "OlmaxQkRopeBwd", "olmax_gemm_glu": "OlmaxGemmGlu",
+            "olmax_glu_bwd": "OlmaxGluBwd", "olmax_embed_fwd": "OlmaxEmbedFwd", "olmax_embed_bwd": "OlmaxEmbedBwd",
+            "olmax_cross_entropy_fwd": "OlmaxCrossEntropyFwd", "olmax_cross_entropy_bwd": "OlmaxCrossEntropyBwd"}
 _registered = False
 
 
@@ -97,7 +107,11 @@ def _attention_vjp():
         B, S, H, D = q.shape
         L = _lib.load()
         L.olmax_attn_bwd_workspace_bytes.restype = ctypes.c_int64
-        nbytes = L.olmax_attn_bwd_workspace_bytes(B, S, H, k.shape[2], D)
+        L.olmax_attn_bwd_workspace_bytes_aligned.restype = ctypes.c_int64
+        # XLA buffers are at least 16-byte aligned and the row strides are heads * D: head_dim 128 takes the
+        # MFMA path, whose scratch is delta only (the general query adds two fp32 [B*S, K*D] accumulators)
+        nbytes = (L.olmax_attn_bwd_workspace_bytes_aligned(B, S, H) if D == 128
+                  else L.olmax_attn_bwd_workspace_bytes(B, S, H, k.shape[2], D))
         dq, dk, dv, _ = jax.ffi.ffi_call(
             "olmax_attn_bwd", (_sds(q.shape, q.dtype), _sds(k.shape, k.dtype), _sds(v.shape, v.dtype), _ws(nbytes)))(
             q, k, v, o, lse, d_o, window=np.int32(window), softcap=np.float32(softcap))
@@ -202,6 +216,166 @@ def _lm_head_vjp():
 
     head.defvjp(fwd, bwd)
     return head
+
+
+# --------------------------------------------------------------------------------------- cross entropy on logits
+_REDUCTIONS = {"mean": 0, "sum": 1, "none": 2}
+
+
+def hip_fused_cross_entropy_loss(logits, labels, *, ignore_index: int = -100, reduction: str = "mean", softcap: float = 0.0):
+    """fused_cross_entropy_loss (src/olmax/nn/functional.py:94-121): (loss, log_normalizer * where) for bf16 or fp32
+    logits [..., V]; the log-normaliser comes back shaped [..., 1] like the reference's keepdims output.  Only the
+    loss is differentiable here (the reference's z-loss users differentiate the normaliser through XLA)."""
+    loss, lse = _cross_entropy_vjp()(logits, labels, int(ignore_index), _REDUCTIONS[reduction], float(softcap))
+    return loss, lse.reshape(*logits.shape[:-1], 1)
+
+
+def hip_cross_entropy_loss(logits, labels, *, ignore_index: int = -100, reduction: str = "mean"):
+    """cross_entropy_loss (src/olmax/nn/functional.py:70-91), reduction "mean" | "sum" | "none"."""
+    return hip_fused_cross_entropy_loss(logits, labels, ignore_index=ignore_index, reduction=reduction)[0]
+
+
+@functools.lru_cache(maxsize=None)
+def _cross_entropy_vjp():
+    jax, jnp = _jax()
+
+    def ws_bytes(T):
+        L = _lib.load()
+        L.olmax_cross_entropy_workspace_bytes.restype = ctypes.c_int64
+        return L.olmax_cross_entropy_workspace_bytes(ctypes.c_int64(T))
+
+    @functools.partial(jax.custom_vjp, nondiff_argnums=(2, 3, 4))
+    def ce(logits, labels, ignore_index, reduction, softcap):
+        return fwd(logits, labels, ignore_index, reduction, softcap)[0]
+
+    def fwd(logits, labels, ignore_index, reduction, softcap):
+        z = logits.reshape(-1, logits.shape[-1])
+        T = z.shape[0]
+        lab = labels.reshape(-1).astype(jnp.int32)
+        loss, lse, _ = jax.ffi.ffi_call(
+            "olmax_cross_entropy_fwd", (_sds((T,) if reduction == 2 else (), jnp.float32), _sds((T,), jnp.float32), _ws(ws_bytes(T))))(
+            z, lab, reduction=np.int32(reduction), ignore_index=np.int32(ignore_index), softcap=np.float32(softcap))
+        if reduction == 2:
+            loss = loss.reshape(labels.shape)
+        return (loss, lse.reshape(labels.shape)), (logits, lab)
+
+    def bwd(ignore_index, reduction, softcap, res, cts):
+        logits, lab = res
+        g = cts[0]  # the normaliser's cotangent is not propagated (see hip_fused_cross_entropy_loss)
+        z = logits.reshape(-1, logits.shape[-1])
+        T = z.shape[0]
+        if reduction == 2:
+            rows = g.reshape(-1).astype(jnp.float32)
+        else:
+            n = jnp.sum(lab != ignore_index).astype(jnp.float32) if reduction == 0 else jnp.float32(1.0)
+            rows = jnp.broadcast_to(g.astype(jnp.float32) / n, (T,))
+        d, _, _ = jax.ffi.ffi_call(
+            "olmax_cross_entropy_bwd", (_sds(z.shape, z.dtype), _sds((T,), jnp.float32), _ws(ws_bytes(T))))(
+            z, lab, rows, ignore_index=np.int32(ignore_index), softcap=np.float32(softcap))
+        return d.reshape(logits.shape), None
+
+    ce.defvjp(fwd, bwd)
+    return ce
+
+
+# --------------------------------------------------------------------------------------- RoPE (+ head-wise QK-norm)
+def hip_rope(x, freqs_cos, freqs_sin, norm_weight=None, eps: float = 1e-5):
+    """RotaryPositionalEmbedding.forward (src/olmax/nn/rope.py:68-80) for x [B, S, H, D] (head_first=False) with the
+    cached tables of get_freqs_cis ([S, D/2] fp32).  With ``norm_weight`` ([D]) the head-wise RMSNorm of
+    src/olmax/nn/attention.py:293-296 runs first in the same kernel."""
+    _, jnp = _jax()
+    w = jnp.ones((x.shape[-1],), x.dtype) if norm_weight is None else norm_weight
+    return _rope_vjp()(x, w, freqs_cos, freqs_sin, norm_weight is not None, float(eps))
+
+
+@functools.lru_cache(maxsize=None)
+def _rope_vjp():
+    jax, jnp = _jax()
+
+    @functools.partial(jax.custom_vjp, nondiff_argnums=(4, 5))
+    def rope(x, w, cos, sin, use_norm, eps):
+        return jax.ffi.ffi_call("olmax_qk_rope_fwd", _sds(x.shape, x.dtype))(
+            x, w, cos.astype(jnp.float32), sin.astype(jnp.float32), use_norm=np.int32(use_norm), eps=np.float32(eps))
+
+    def fwd(x, w, cos, sin, use_norm, eps):
+        return rope(x, w, cos, sin, use_norm, eps), (x, w, cos, sin)
+
+    def bwd(use_norm, eps, res, dy):
+        x, w, cos, sin = res
+        dx, dw = jax.ffi.ffi_call("olmax_qk_rope_bwd", (_sds(x.shape, x.dtype), _sds(w.shape, jnp.float32)))(
+            dy, x, w, cos.astype(jnp.float32), sin.astype(jnp.float32), use_norm=np.int32(use_norm), eps=np.float32(eps))
+        return dx, dw.astype(w.dtype), jnp.zeros_like(cos), jnp.zeros_like(sin)
+
+    rope.defvjp(fwd, bwd)
+    return rope
+
+
+# --------------------------------------------------------------------------------------- gated MLP input half
+_ACTS = {"silu": 0, "gelu": 1}
+
+
+def hip_gated_mlp_in(x, gate_weight, up_weight, activation: str = "silu"):
+    """act(gate_proj(x)) * up_proj(x) of GatedMLP.forward (src/olmax/nn/mlp.py:69-73) as ONE GEMM over
+    [Wgate; Wup] with the activation in its epilogue; the down projection stays ``hip_linear``.  (The Equinox
+    module owns two Linear layers, so the two weights are concatenated per call; a module that stores them
+    adjacent, as the flat layout of ``HipTrainStep`` does, skips that copy.)"""
+    return _gated_vjp()(x, gate_weight, up_weight, _ACTS[activation])
+
+
+@functools.lru_cache(maxsize=None)
+def _gated_vjp():
+    jax, jnp = _jax()
+    linear = _linear_vjp()
+
+    @functools.partial(jax.custom_vjp, nondiff_argnums=(3,))
+    def gated(x, wg, wu, act):
+        return fwd(x, wg, wu, act)[0]
+
+    def fwd(x, wg, wu, act):
+        F = wg.shape[0]
+        w = jnp.concatenate([wg, wu], axis=0)
+        out, gu = jax.ffi.ffi_call("olmax_gemm_glu", (_sds((*x.shape[:-1], F), x.dtype), _sds((*x.shape[:-1], 2 * F), x.dtype)))(
+            x, w, act=np.int32(act))
+        return out, (x, w, gu)
+
+    def bwd(act, res, dh):
+        x, w, gu = res
+        F = w.shape[0] // 2
+        dgu = jax.ffi.ffi_call("olmax_glu_bwd", _sds(gu.shape, gu.dtype))(gu, dh, act=np.int32(act))
+        x2, dgu2 = x.reshape(-1, x.shape[-1]), dgu.reshape(-1, 2 * F)
+        dx = jax.ffi.ffi_call("olmax_gemm", _sds(x.shape, x.dtype))(dgu2, w, a_layout=np.int32(0), b_layout=np.int32(1))
+        dw = jax.ffi.ffi_call("olmax_gemm", _sds(w.shape, w.dtype))(dgu2, x2, a_layout=np.int32(1), b_layout=np.int32(1))
+        return dx, dw[:F], dw[F:]
+
+    gated.defvjp(fwd, bwd)
+    return gated
+
+
+# --------------------------------------------------------------------------------------- embedding
+def hip_embedding(weight, ids):
+    """Embedding.forward (src/olmax/nn/embedding.py:30-32): rows of weight [V, d] (bf16) for integer ids of any
+    shape; the backward is the fp32 scatter-add, cast back to the weight's dtype."""
+    return _embedding_vjp()(weight, ids)
+
+
+@functools.lru_cache(maxsize=None)
+def _embedding_vjp():
+    jax, jnp = _jax()
+
+    @jax.custom_vjp
+    def embed(w, ids):
+        return jax.ffi.ffi_call("olmax_embed_fwd", _sds((*ids.shape, w.shape[1]), w.dtype))(ids.astype(jnp.int32), w)
+
+    def fwd(w, ids):
+        return embed(w, ids), (w, ids)
+
+    def bwd(res, dh):
+        w, ids = res
+        dw = jax.ffi.ffi_call("olmax_embed_bwd", _sds(w.shape, jnp.float32))(ids.astype(jnp.int32), dh)
+        return dw.astype(w.dtype), None
+
+    embed.defvjp(fwd, bwd)
+    return embed
 
 
 # --------------------------------------------------------------------------------------- optimizer

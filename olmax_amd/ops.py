@@ -239,25 +239,30 @@ def attn_bwd(q, k, v, o, lse, do, *, B: int, S: int, H: int, KH: int, D: int, wi
 
 # ----------------------------------------------------------------------------- cross entropy / LM head
 def cross_entropy(logits, labels, *, ignore_index: int = -100, softcap: float = 0.0, want_grad: bool = True,
-                  inplace: bool = False, dloss: float = 1.0):
-    """logits [T, V] bf16 or fp32, labels [T] int32 -> (loss scalar tensor, dlogits or None, lse [T])."""
-    _need_gpu(logits, labels)
+                  inplace: bool = False, dloss: float = 1.0, reduction: str = "mean", dloss_rows=None):
+    """logits [T, V] bf16 or fp32, labels [T] int32 -> (loss, dlogits or None, lse [T]);
+    reduction "mean" | "sum" | "none" as cross_entropy_loss (src/olmax/nn/functional.py:70-91):
+    loss is a scalar tensor, or [T] for "none" (whose per-row cotangent is dloss * dloss_rows)."""
+    _need_gpu(logits, labels, dloss_rows)
     logits = _rows2d(logits)
     assert labels.dtype == torch.int32
+    red = {"mean": 0, "sum": 1, "none": 2}[reduction]
     T, V = logits.shape
     L = _L()
     L.olmax_cross_entropy_workspace_bytes.restype = i64
     nbytes = L.olmax_cross_entropy_workspace_bytes(i64(T))
     ws = torch.empty(nbytes, device=logits.device, dtype=torch.uint8)
-    loss = torch.empty((), device=logits.device, dtype=torch.float32)
+    loss = torch.empty((T,) if red == 2 else (), device=logits.device, dtype=torch.float32)
     lse = torch.empty(T, device=logits.device, dtype=torch.float32)
     d = None
     if want_grad:
         d = logits if inplace else torch.empty_like(logits)
-    check(L.olmax_cross_entropy(stream_ptr(), ptr(logits), ptr(d), ptr(labels), ptr(loss), ptr(lse), ptr(ws),
-                                i64(nbytes), i64(T), i32(V), i64(logits.stride(0)),
-                                i64(0 if d is None else d.stride(0)), i32(1 if logits.dtype == torch.float32 else 0),
-                                i32(ignore_index), f32(softcap), f32(dloss)))
+    if dloss_rows is not None:
+        assert dloss_rows.dtype == torch.float32 and dloss_rows.numel() == T and dloss_rows.is_contiguous()
+    check(L.olmax_cross_entropy_reduce(stream_ptr(), ptr(logits), ptr(d), ptr(labels), ptr(loss), ptr(lse), ptr(dloss_rows),
+                                       ptr(ws), i64(nbytes), i64(T), i32(V), i64(logits.stride(0)),
+                                       i64(0 if d is None else d.stride(0)), i32(1 if logits.dtype == torch.float32 else 0),
+                                       i32(ignore_index), f32(softcap), f32(dloss), i32(red)))
     return loss, d, lse
 
 

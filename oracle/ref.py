@@ -230,8 +230,8 @@ def attention_bwd(q, k, v, o, lse, do, *, window=None, softcap: float = 0.0, rt=
 
 # --------------------------------------------------------------------------- cross entropy
 def cross_entropy_fwd(logits: Tensor, labels: Tensor, ignore_index: int = -100,
-                      softcap: float = 0.0):
-    """src/olmax/nn/functional.py:70-91, reduction="mean".
+                      softcap: float = 0.0, reduction: str = "mean"):
+    """src/olmax/nn/functional.py:70-91; reduction "mean" (default), "sum" or "none" (:84-91).
 
     Quirks kept: a label outside [0, V) that is not ignore_index has an all-zero one-hot, so
     its loss is 0 but it still counts in the mean's denominator; ignore_index rows count in
@@ -247,13 +247,21 @@ def cross_entropy_fwd(logits: Tensor, labels: Tensor, ignore_index: int = -100,
     tgt = torch.gather(z, -1, labels.clamp(0, V - 1)[..., None].long())[..., 0]
     per = torch.where(where & inrange, lse - tgt, torch.zeros_like(lse))
     n = where.sum()
-    loss = per.sum() / n
+    if reduction == "mean":
+        loss = per.sum() / n
+    elif reduction == "sum":
+        loss = per.sum()
+    elif reduction == "none":
+        loss = per
+    else:
+        raise ValueError(reduction)
     return loss, lse, n
 
 
 def cross_entropy_bwd(logits: Tensor, labels: Tensor, ignore_index: int = -100,
-                      softcap: float = 0.0, dloss: float = 1.0) -> Tensor:
-    """dlogits_i = (softmax_i - onehot_i) / n for counted in-range rows, 0 otherwise."""
+                      softcap: float = 0.0, dloss=1.0, reduction: str = "mean") -> Tensor:
+    """dlogits_i = (softmax_i - onehot_i) * dloss / n for counted in-range rows, 0 otherwise
+    ("sum": no division by n; "none": dloss is the per-row cotangent [T])."""
     V = logits.shape[-1]
     z = logits
     t = None
@@ -265,7 +273,13 @@ def cross_entropy_bwd(logits: Tensor, labels: Tensor, ignore_index: int = -100,
     n = where.sum()
     p = torch.softmax(z, -1)
     oh = torch.nn.functional.one_hot(labels.clamp(0, V - 1).long(), V).to(z.dtype)
-    d = (p - oh) * (where & inrange)[..., None].to(z.dtype) * (dloss / n)
+    if reduction == "mean":
+        scale = dloss / n
+    elif reduction == "sum":
+        scale = dloss
+    else:
+        scale = torch.as_tensor(dloss, dtype=z.dtype).reshape(-1, 1) * torch.ones(z.shape[0], 1, dtype=z.dtype)
+    d = (p - oh) * (where & inrange)[..., None].to(z.dtype) * scale
     if t is not None:
         d = d * (1.0 - t * t)
     return d

@@ -50,7 +50,9 @@ def test_adapter_calls_match_the_header():
     header, adapter = _strip_comments(HEADER), _strip_comments(ADAPTER)
     called = sorted(set(re.findall(r"\b(olmax_[a-z0-9_]+)\s*\(", adapter)))
     assert {"olmax_attn_fwd", "olmax_attn_bwd", "olmax_rmsnorm_fwd", "olmax_rmsnorm_bwd", "olmax_gemm_bf16",
-            "olmax_lmhead_ce", "olmax_adamw_dev", "olmax_model_train_step"} <= set(called)
+            "olmax_lmhead_ce", "olmax_adamw_dev", "olmax_model_train_step", "olmax_qk_rope_fwd", "olmax_qk_rope_bwd",
+            "olmax_gemm_glu_bf16", "olmax_glu_bwd", "olmax_embed_fwd", "olmax_embed_bwd", "olmax_cross_entropy_reduce",
+            "olmax_model_layout", "olmax_model_num_params", "olmax_model_workspace_bytes"} <= set(called)
     for name in called:
         decl = _calls(header, name)
         assert len(decl) == 1, f"{name} is not declared exactly once in olmax_hip.h"
@@ -61,7 +63,7 @@ def test_adapter_calls_match_the_header():
 def test_every_registered_target_has_a_handler_symbol():
     src = (ROOT / "olmax_amd" / "jax_ffi.py").read_text()
     targets = dict(re.findall(r'"(olmax_[a-z_]+)":\s*"(Olmax[A-Za-z]+)"', src))
-    assert len(targets) == 8
+    assert len(targets) == 16
     defined = set(re.findall(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\(\s*(Olmax[A-Za-z]+)", ADAPTER))
     assert set(targets.values()) == defined
     used = set(re.findall(r'ffi_call\(\s*"(olmax_[a-z_]+)"', src))

@@ -430,6 +430,35 @@ def test_cross_entropy_in_place_equals_out_of_place(V, f32):
         assert abs(l0.item() - (lse0 - zl).mean().item()) < 1e-4
 
 
+@pytest.mark.parametrize("T,V,f32", [(33, 4096, False), (7, 100352, False), (5, 1003, False), (9, 4104, True), (3, 262144, False)])
+def test_cross_entropy_sum_and_none_reductions(T, V, f32):
+    """reduction "sum" and "none" of cross_entropy_loss (src/olmax/nn/functional.py:84-91), forward and
+    backward (scalar cotangent, and per-row cotangents for "none"), against the oracle."""
+    ops = _ops()
+    say(f"ce reductions T{T} V{V} f32{f32}")
+    g = torch.Generator().manual_seed(2)
+    logits = torch.randn(T, V, generator=g) * 3
+    logits = logits if f32 else logits.to(BF)
+    labels = torch.randint(0, V, (T,), generator=g, dtype=torch.int32)
+    labels[1] = -100
+    labels[2] = V
+    tol = 1e-4 if f32 else 1e-2
+    loss, d, _ = ops.cross_entropy(logits.cuda(), labels.cuda(), reduction="sum", dloss=0.5)
+    wl = ref.cross_entropy_fwd(logits.double(), labels.long(), reduction="sum")[0]
+    assert abs(loss.item() - wl.item()) < 2e-3 * max(1.0, abs(wl.item()))
+    check_close(d, ref.cross_entropy_bwd(logits.double(), labels.long(), dloss=0.5, reduction="sum"), "dlogits sum", tol=tol)
+    w = torch.randn(T, generator=g)
+    loss, d, _ = ops.cross_entropy(logits.cuda(), labels.cuda(), reduction="none", dloss_rows=w.cuda())
+    wl = ref.cross_entropy_fwd(logits.double(), labels.long(), reduction="none")[0]
+    assert loss.shape == (T,) and (loss.cpu().double() - wl).abs().max() < 2e-3
+    assert loss[1].item() == 0 and loss[2].item() == 0
+    check_close(d, ref.cross_entropy_bwd(logits.double(), labels.long(), dloss=w.double(), reduction="none"), "dlogits none", tol=tol)
+    # mean == sum / counted rows
+    lm, _, _ = ops.cross_entropy(logits.cuda(), labels.cuda(), want_grad=False)
+    ls, _, _ = ops.cross_entropy(logits.cuda(), labels.cuda(), want_grad=False, reduction="sum")
+    assert abs(lm.item() * (T - 1) - ls.item()) < 1e-4 * abs(ls.item())
+
+
 def test_cross_entropy_reference_invariants():
     """src/test/nn/functional_test.py:10-18: an appended ignore_index row leaves the mean unchanged."""
     ops = _ops()

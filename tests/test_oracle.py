@@ -164,6 +164,29 @@ def test_cross_entropy():
     assert d.sum(-1).abs().max() < 1e-12 and d[2].abs().max() == 0
 
 
+def test_cross_entropy_sum_and_none_reductions():
+    """src/olmax/nn/functional.py:84-91 against torch's own reductions, forward and backward."""
+    g = torch.Generator().manual_seed(4)
+    T, V = 9, 23
+    logits = torch.randn(T, V, generator=g, dtype=D64)
+    labels = torch.randint(0, V, (T,), generator=g)
+    labels[2] = -100
+    for red in ("sum", "none"):
+        got = ref.cross_entropy_fwd(logits, labels, reduction=red)[0]
+        want = F.cross_entropy(logits, labels, ignore_index=-100, reduction=red)
+        assert torch.allclose(got, want, atol=1e-12)
+    lg = logits.clone().requires_grad_(True)
+    (gs,) = torch.autograd.grad(F.cross_entropy(lg, labels, ignore_index=-100, reduction="sum") * 0.5, lg)
+    assert torch.allclose(ref.cross_entropy_bwd(logits, labels, dloss=0.5, reduction="sum"), gs, atol=1e-12)
+    w = torch.randn(T, generator=g, dtype=D64)
+    (gn,) = torch.autograd.grad((F.cross_entropy(lg, labels, ignore_index=-100, reduction="none") * w).sum(), lg)
+    assert torch.allclose(ref.cross_entropy_bwd(logits, labels, dloss=w, reduction="none"), gn, atol=1e-12)
+    # out-of-range label (one_hot gives an all-zero row): zero loss and gradient in every reduction
+    labels[4] = V
+    per = ref.cross_entropy_fwd(logits, labels, reduction="none")[0]
+    assert per[4] == 0 and per[2] == 0 and ref.cross_entropy_bwd(logits, labels, reduction="sum")[4].abs().max() == 0
+
+
 def test_cross_entropy_out_of_range_label_quirk():
     """label == V (made by the synthetic loader when input == V-1): zero loss, zero grad, but
     the row still counts in the mean (one_hot gives zeros; `where` is labels != -100)."""
