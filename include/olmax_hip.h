@@ -103,6 +103,15 @@ int32_t olmax_gemm_glu_bf16(olmax_stream_t stream, const void* X, const void* W,
                             int32_t M, int32_t F, int32_t K, int64_t ldx, int64_t ldw, int64_t ldgu,
                             int64_t ldact, int32_t act);
 
+/* The same projection re-run in the backward pass of a block that kept nothing (full-block recompute,
+ * src/olmax/activation_checkpointing.py:71-80): from X, W and dact = d loss / d(act(gate) * up) it writes
+ * act_out [M, F] (the operand of the down projection's weight gradient) and dgu_out [M, 2F] =
+ * d gate | d up; gate | up stay in the accumulators.  Results equal olmax_gemm_glu_bf16 followed by
+ * olmax_glu_bwd bit for bit (the path taken, through dgu_out as scratch, when the shape does not fit). */
+int32_t olmax_gemm_glu_bwd_bf16(olmax_stream_t stream, const void* X, const void* W, const void* dact, void* act_out,
+                                void* dgu_out, int32_t M, int32_t F, int32_t K, int64_t ldx, int64_t ldw,
+                                int64_t lddact, int64_t ldact, int64_t lddgu, int32_t act);
+
 /* ---- q|k|v projection with the rotary embedding fused into the GEMM epilogue:
  * MultiheadSelfAttention.forward, src/olmax/nn/attention.py:270-274 (projections) and :298-300
  * (RoPE on q and k, src/olmax/nn/rope.py:99-115), for recipes without QK-norm.

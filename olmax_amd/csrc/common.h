@@ -144,6 +144,16 @@ __device__ __forceinline__ float act_gelu(float g) {
   return 0.5f * g * (1.f + fast_tanh(GELU_C * (g + 0.044715f * g * g * g)));
 }
 
+// derivatives of the two activations (the backward of act(gate) * up)
+__device__ __forceinline__ float act_silu_grad(float g) {
+  const float s = 1.f / (1.f + __expf(-g));
+  return s * (1.f + g * (1.f - s));
+}
+__device__ __forceinline__ float act_gelu_grad(float g) {
+  const float t = fast_tanh(GELU_C * (g + 0.044715f * g * g * g));
+  return 0.5f * (1.f + t) + 0.5f * g * (1.f - t * t) * GELU_C * (1.f + 3.f * 0.044715f * g * g);
+}
+
 // elementwise.hip, library-internal: olmax_adamw_dscale with the grid size (workgroups) exposed.
 int olmax_adamw_grid(hipStream_t stream, float* p, const void* g, float* m, float* v, void* shadow_bf16, int64_t n,
                      int32_t grad_is_bf16, float lr, float b1, float b2, float eps, float wd, int64_t step,

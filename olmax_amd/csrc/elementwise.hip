@@ -14,15 +14,6 @@
 
 namespace {
 
-__device__ __forceinline__ float act_silu_grad(float g) {
-  const float s = 1.f / (1.f + __expf(-g));
-  return s * (1.f + g * (1.f - s));
-}
-__device__ __forceinline__ float act_gelu_grad(float g) {
-  const float t = fast_tanh(GELU_C * (g + 0.044715f * g * g * g));
-  return 0.5f * (1.f + t) + 0.5f * g * (1.f - t * t) * GELU_C * (1.f + 3.f * 0.044715f * g * g);
-}
-
 // gate/up are column blocks of one [T, ld] buffer (or separate buffers); out [T, F].
 template <bool GELU>
 __global__ __launch_bounds__(256) void glu_fwd_kernel(const bf16* __restrict__ gate,

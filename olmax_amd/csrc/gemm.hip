@@ -64,6 +64,13 @@ std::mutex g_prof_mu;
 // same 32 features; the epilogue writes act = f(gate) * up ([M, F], leading dimension ldr) and,
 // when Cv is given, gate|up ([M, 2F]) as the plain GEMM would.  N is F in that mode.
 //
+// EPI == 4 / 5 (silu / tanh-gelu) is the same projection run in the BACKWARD pass of a block whose
+// forward kept nothing: gate and up are recomputed in the accumulators and, with the gradient of
+// the activation output (dact [M, F], passed through the cos_t pointer with its row stride in
+// seq_len), leave the kernel as act = f(gate) * up (R, for the down projection's weight gradient)
+// and d gate | d up (Cv [M, 2F]) -- gate | up never reach memory and no separate GLU backward
+// kernel runs.  Same roundings as olmax_gemm_glu_bf16 followed by olmax_glu_bwd.
+//
 // EPI == 3 is the fused q|k|v projection + rotary embedding: columns below rope_cols are heads of
 // 128 that leave the kernel rotated (out = x cos + rotate_half(x) sin in fp32 on the bf16-rounded
 // projection, as the separate RoPE kernel computes it); a wave's 64 columns are one half of a
@@ -75,7 +82,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
     const bf16* __restrict__ R, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
     int64_t ldr, int tiles_m, int tiles_n, int c_vec, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int seq_len, int rope_cols, int order) {
-  constexpr int GLU = (EPI == 1 || EPI == 2) ? EPI : 0;
+  constexpr int GLU = (EPI == 1 || EPI == 2) ? EPI : (EPI == 4 ? 1 : (EPI == 5 ? 2 : 0));
+  constexpr bool GLU_BWD = EPI == 4 || EPI == 5;
   constexpr bool ROPE = EPI == 3;
   static_assert(EPI == 0 || (BN == 256 && WN == 64 && B_KC && !HAS_RES && !OUT_F32), "fused epilogues: 256-wide NT tiles only");
   constexpr int NW = (BM / WM) * (BN / WN);
@@ -411,11 +419,24 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
       // Whole-line stores through LDS.  A wave's 128 x 32 features are half a line per row, so the
       // block's 256 x 128 output is staged wave by wave (64-byte rows, 16-byte chunks XOR-swizzled
       // by (row >> 2) & 3) and written out by rows: wave w takes rows 32w .. 32w+31, four rows of
-      // 256 B per instruction.  First act, then (when kept for the backward pass) gate and up.
+      // 256 B per instruction.  First act, then (when kept for the backward pass) gate and up, or,
+      // in the backward form, d gate and d up.
       constexpr int REG = WM * 64;  // bytes of one wave's staging region
+      // backward form: this lane's gradients of the activation output, in accumulator layout
+      // (8 bytes = its 4 features of one row), requested before the barrier that they ride out
+      Pack4 dd[GLU_BWD ? TM : 1][2];
+      if (GLU_BWD) {
+        const bf16* dact = reinterpret_cast<const bf16*>(cos_t);
+        const int64_t lddact = seq_len;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++)
+            dd[i][j].u = *reinterpret_cast<const u32x2*>(dact + (int64_t)(m0 + wm * WM + i * 16 + l16e) * lddact + n0 + wn * 32 + j * 16 + g16e * 4);
+      }
       __syncthreads();              // every wave is done reading the operand stages
 #pragma unroll 1
-      for (int pass = 0; pass < (gu ? 2 : 1); pass++) {
+      for (int pass = 0; pass < ((gu || GLU_BWD) ? 2 : 1); pass++) {
         if (pass) __syncthreads();  // the previous pass has been read back
 #pragma unroll
         for (int i = 0; i < TM; i++)
@@ -430,8 +451,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
               pg.e[r] = f2bf(acc[i][j][r]);
               pu.e[r] = f2bf(acc[i][j + 2][r]);
               const float gf = bf2f(pg.e[r]);
-              const float a = bf2f(f2bf(GLU == 2 ? act_gelu(gf) : act_silu(gf)));
-              pa.e[r] = f2bf(a * bf2f(pu.e[r]));
+              const float fg = GLU == 2 ? act_gelu(gf) : act_silu(gf);
+              pa.e[r] = f2bf(bf2f(f2bf(fg)) * bf2f(pu.e[r]));
+              if (GLU_BWD) {  // d gate = dact * up * f'(gate), d up = dact * f(gate)
+                const float df = bf2f(dd[GLU_BWD ? i : 0][j].e[r]);
+                pg.e[r] = f2bf(df * bf2f(pu.e[r]) * (GLU == 2 ? act_gelu_grad(gf) : act_silu_grad(gf)));
+                pu.e[r] = f2bf(df * fg);
+              }
             }
             if (pass == 0) {
               *reinterpret_cast<u32x2*>(dst) = pa.u;
@@ -456,6 +482,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) GEMM_VGPR_CAP void gemm
       }
       return;
     }
+    if (GLU_BWD) return;  // the backward form is only launched with whole-line stores
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -678,11 +705,12 @@ int launch_tile(hipStream_t s, const bf16* A, const bf16* B, void* C, const bf16
   return OLMAX_OK;
 }
 
-template <int GLU>
+// EPI 1 / 2: forward form (gu optional); 4 / 5: backward form (dact given, gu = d gate | d up)
+template <int EPI>
 int launch_glu(hipStream_t s, const bf16* A, const bf16* B, bf16* gu, bf16* act, int M, int F, int K, int64_t lda,
-               int64_t ldb, int64_t ldgu, int64_t ldact) {
+               int64_t ldb, int64_t ldgu, int64_t ldact, const bf16* dact = nullptr, int64_t lddact = 0) {
   constexpr int SMEM = 2 * (256 + 256) * BK * 2;
-  auto kern = gemm_bf16_kernel<256, 256, 128, 64, true, true, false, false, GLU>;
+  auto kern = gemm_bf16_kernel<256, 256, 128, 64, true, true, false, false, EPI>;
   static std::once_flag attr_once;  // per instantiation
   std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM); });
   const int tm = M / 256, tn = F / 128;
@@ -697,11 +725,11 @@ int launch_glu(hipStream_t s, const bf16* A, const bf16* B, bf16* gu, bf16* act,
                     : ((((uintptr_t)act) & 7) == 0 && ldact % 4 == 0 && (!gu || ((((uintptr_t)gu) & 7) == 0 && ldgu % 4 == 0 && F % 4 == 0)));
   const int order = tile_order(tm, tn, true, true, 2 * F, K);
   hipLaunchKernelGGL(kern, dim3(order_grid(order, tm, tn)), dim3(512), SMEM, s, A, B, (void*)gu, (const bf16*)act, M, F, K, lda, ldb,
-                     ldgu, ldact, tm, tn, c_vec, (const float*)nullptr, (const float*)nullptr, 1, 0, order);
+                     ldgu, ldact, tm, tn, c_vec, reinterpret_cast<const float*>(dact), (const float*)nullptr, (int)lddact, 0, order);
   if (g_prof_on) {
     (void)hipEventRecord(rec.e1, s);
     rec.flops = 4.0 * M * F * K;
-    rec.bytes = 2.0 * ((double)M * K + 2.0 * F * K + (double)M * F * (gu ? 3 : 1));
+    rec.bytes = 2.0 * ((double)M * K + 2.0 * F * K + (double)M * F * ((gu ? 3 : 1) + (dact ? 1 : 0)));
     rec.key = 256 | (1 << 12) | (1 << 13) | (1 << 16);
     rec.M = M; rec.N = 2 * F; rec.K = K;
     std::lock_guard<std::mutex> lk(g_prof_mu);
@@ -960,4 +988,39 @@ extern "C" int32_t olmax_gemm_glu_bf16(hipStream_t stream, const void* X, const 
   int rc = olmax_gemm_bf16(stream, X, W, gu_out, nullptr, M, 2 * F, K, ldx, ldw, ldgu, 0, 0, 0, 0);
   if (rc) return rc;
   return olmax_glu_fwd(stream, gu_out, (const bf16*)gu_out + F, act_out, M, F, ldgu, ldgu, ldact, act);
+}
+
+extern "C" int32_t olmax_glu_bwd(hipStream_t stream, const void* gate, const void* up, const void* dh, void* dgate, void* dup,
+                                 int64_t T, int32_t F, int64_t ldg, int64_t ldu, int64_t lddh, int64_t lddg, int64_t lddu,
+                                 int32_t act);
+
+// The gated-MLP input projection re-run inside the backward pass (full-block recompute): from X, W = [Wgate; Wup] and
+// dact = d loss / d (act(gate) * up) it produces act_out [M, F] (what the down projection's weight gradient needs) and
+// dgu_out [M, 2F] = d gate | d up, without gate | up ever being written.  Equals olmax_gemm_glu_bf16 followed by
+// olmax_glu_bwd, which is also the path taken (through dgu_out as scratch for gate | up) when the shape does not
+// fit the tile.
+extern "C" int32_t olmax_gemm_glu_bwd_bf16(hipStream_t stream, const void* X, const void* W, const void* dact, void* act_out,
+                                           void* dgu_out, int32_t M, int32_t F, int32_t K, int64_t ldx, int64_t ldw,
+                                           int64_t lddact, int64_t ldact, int64_t lddgu, int32_t act) {
+  OLMAX_CHECK(X && W && dact && act_out && dgu_out, OLMAX_ERR_ARG, "olmax_gemm_glu_bwd_bf16: null operand");
+  OLMAX_CHECK(M > 0 && F > 0 && K > 0, OLMAX_ERR_SHAPE, "olmax_gemm_glu_bwd_bf16: M,F,K must be positive (got %d,%d,%d)", M, F, K);
+  OLMAX_CHECK(act == 0 || act == 1, OLMAX_ERR_ARG, "olmax_gemm_glu_bwd_bf16: act must be 0 (silu) or 1 (gelu-tanh)");
+  OLMAX_CHECK(ldx >= K && ldw >= K && ldact >= F && lddact >= F && lddgu >= 2 * (int64_t)F, OLMAX_ERR_SHAPE,
+              "olmax_gemm_glu_bwd_bf16: leading dimension smaller than row length");
+  const bool fits = aligned16(X) && aligned16(W) && ldx % 8 == 0 && ldw % 8 == 0 && K % BK == 0 && M % 256 == 0 &&
+                    F % 128 == 0 && (int64_t)(M / 256) * (F / 128) >= 128 && !g_force_tile.load(std::memory_order_relaxed) &&
+                    aligned16(act_out) && ldact % 8 == 0 && aligned16(dgu_out) && lddgu % 8 == 0 &&
+                    ((((uintptr_t)dact) & 7) == 0) && lddact % 4 == 0 && lddact < (1ll << 31);
+  if (fits) {
+    if (act == 0)
+      return launch_glu<4>(stream, (const bf16*)X, (const bf16*)W, (bf16*)dgu_out, (bf16*)act_out, M, F, K, ldx, ldw, lddgu, ldact,
+                           (const bf16*)dact, lddact);
+    return launch_glu<5>(stream, (const bf16*)X, (const bf16*)W, (bf16*)dgu_out, (bf16*)act_out, M, F, K, ldx, ldw, lddgu, ldact,
+                         (const bf16*)dact, lddact);
+  }
+  // unfused: gate | up into dgu_out, then the elementwise backward in place over it
+  int rc = olmax_gemm_glu_bf16(stream, X, W, dgu_out, act_out, M, F, K, ldx, ldw, lddgu, ldact, act);
+  if (rc) return rc;
+  return olmax_glu_bwd(stream, dgu_out, (const bf16*)dgu_out + F, dact, dgu_out, (bf16*)dgu_out + F, M, F, lddgu, lddgu, lddact, lddgu,
+                       lddgu, act);
 }

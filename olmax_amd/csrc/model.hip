@@ -132,7 +132,7 @@ int lin_dw(hipStream_t s, const bf16* dy, int64_t lddy, const bf16* x, int64_t l
 // the backward pass, so the GEMM / norm that only produces it is skipped.
 // Points inside a block's backward pass at which the overlapped train step may start queued
 // optimizer work on its second stream (set only while olmax_model_train_step runs).
-enum { POINT_RECOMPUTE_ATTN = 1, POINT_ATTN_BWD = 2 };
+enum { POINT_RECOMPUTE_ATTN = 1, POINT_ATTN_BWD = 2, POINT_AFTER_DACT = 3 };
 struct StepHook {
   int (*fn)(void* ctx, int point) = nullptr;
   void* ctx = nullptr;
@@ -140,9 +140,12 @@ struct StepHook {
 thread_local StepHook g_hook;
 inline int hook_point(int point) { return g_hook.fn ? g_hook.fn(g_hook.ctx, point) : OLMAX_OK; }
 
+// defer_mlp (recompute of a pre-norm block only): stop after the MLP's input norm; the gated
+// projection is re-run by the backward pass itself, fused with the GLU backward
+// (olmax_gemm_glu_bwd_bf16), so gate | up are never written.
 int block_forward(hipStream_t s, const olmax_model_config* c, const olmax_block_weights* w, int window,
                   const float* cos_t, const float* sin_t, const bf16* x, bf16* y, const Acts& a,
-                  bool need_y = true, bool save_gu = true) {
+                  bool need_y = true, bool save_gu = true, bool defer_mlp = false) {
   const Dims m = dims_of(c);
   const int lt = c->layer_type;
   const float eps = c->eps;
@@ -194,6 +197,7 @@ int block_forward(hipStream_t s, const olmax_model_config* c, const olmax_block_
     RC(olmax_rmsnorm_fwd(s, a.h, lt == 0 ? w->mlp_norm : w->mlp_in_norm, a.hn, m.T, m.d, m.d, m.d, eps));
     mlp_in = a.hn;
   }
+  if (defer_mlp) return OLMAX_OK;
   // gate|up projection with the activation in the GEMM epilogue; gate|up themselves are only
   // written when a backward pass will read them (a.gu doubles as scratch for odd shapes)
   const bool fused_shape = m.T % 256 == 0 && m.F % 128 == 0 && m.d % 64 == 0 && (m.T / 256) * (m.F / 128) >= 128;
@@ -250,14 +254,22 @@ int attn_backward(hipStream_t s, const olmax_model_config* c, const olmax_block_
 }
 
 // MLP part: d_mlp_out [T,d] -> grads of wdown, wgu and d(mlp input) into `dxin` (+ res).
+// deferred: the block's recompute stopped before the MLP and d act = d_mlp_out Wdown is already in
+// t.dact; the gated projection runs here in its backward form (act for the down projection's
+// weight gradient, d gate | d up straight from the accumulators).
 int mlp_backward(hipStream_t s, const olmax_model_config* c, const olmax_block_weights* w,
                  const olmax_block_grads* g, const bf16* mlp_in, const bf16* d_mlp_out, bf16* dxin,
-                 const bf16* res_for_dx, const Acts& a, const Tmp& t) {
+                 const bf16* res_for_dx, const Acts& a, const Tmp& t, bool deferred = false) {
   const Dims m = dims_of(c);
-  RC(lin_dx(s, d_mlp_out, m.d, w->wdown, m.F, m.d, t.dact, m.F, nullptr, 0, m.T));
+  if (deferred) {
+    RC(olmax_gemm_glu_bwd_bf16(s, mlp_in, w->wgu, t.dact, a.act, t.dgu, (int)m.T, m.F, m.d, m.d, m.d, m.F, m.F, 2 * m.F, c->act));
+  } else {
+    RC(lin_dx(s, d_mlp_out, m.d, w->wdown, m.F, m.d, t.dact, m.F, nullptr, 0, m.T));
+  }
   RC(lin_dw(s, d_mlp_out, m.d, a.act, m.F, m.F, m.d, g->wdown, m.T));
-  RC(olmax_glu_bwd(s, a.gu, a.gu + m.F, t.dact, t.dgu, t.dgu + m.F, m.T, m.F, 2 * m.F, 2 * m.F, m.F, 2 * m.F, 2 * m.F,
-                   c->act));
+  if (!deferred)
+    RC(olmax_glu_bwd(s, a.gu, a.gu + m.F, t.dact, t.dgu, t.dgu + m.F, m.T, m.F, 2 * m.F, 2 * m.F, m.F, 2 * m.F, 2 * m.F,
+                     c->act));
   RC(lin_dx(s, t.dgu, 2 * m.F, w->wgu, m.d, 2 * m.F, dxin, m.d, res_for_dx, m.d, m.T));
   RC(lin_dw(s, t.dgu, 2 * m.F, mlp_in, m.d, m.d, 2 * m.F, g->wgu, m.T));
   return OLMAX_OK;
@@ -265,12 +277,12 @@ int mlp_backward(hipStream_t s, const olmax_model_config* c, const olmax_block_w
 
 int block_backward(hipStream_t s, const olmax_model_config* c, const olmax_block_weights* w,
                    const olmax_block_grads* g, int window, const float* cos_t, const float* sin_t,
-                   const bf16* x, const bf16* dy, bf16* dx, const Acts& a, const Tmp& t) {
+                   const bf16* x, const bf16* dy, bf16* dx, const Acts& a, const Tmp& t, bool mlp_deferred = false) {
   const Dims m = dims_of(c);
   const int lt = c->layer_type;
   const float eps = c->eps;
   if (lt == 0) {
-    RC(mlp_backward(s, c, w, g, a.hn, dy, t.d1, nullptr, a, t));                                       // d1 = d hn
+    RC(mlp_backward(s, c, w, g, a.hn, dy, t.d1, nullptr, a, t, mlp_deferred));                         // d1 = d hn
     RC(olmax_rmsnorm_bwd(s, a.h, w->mlp_norm, t.d1, dy, t.d2, g->mlp_norm, m.T, m.d, m.d, m.d, m.d, m.d, eps));  // d2 = dh
     RC(attn_backward(s, c, w, g, window, cos_t, sin_t, a.xn, t.d2, t.d1, nullptr, a, t));              // d1 = d xn
     RC(olmax_rmsnorm_bwd(s, x, w->attn_norm, t.d1, t.d2, dx, g->attn_norm, m.T, m.d, m.d, m.d, m.d, m.d, eps));
@@ -500,11 +512,20 @@ int model_run(hipStream_t s, const olmax_model_config* c, const int32_t* windows
     Arena aa(w.acts_base + (keep ? (int64_t)l * w.acts_stride : 0));
     Acts acts = carve_acts(c, aa);
     const bf16* xin = w.xs + (int64_t)l * Td;
+    // Pre-norm blocks under recompute: the gradient of the activation output only needs dY and
+    // Wdown, so it goes first; the recompute then stops at the MLP's input norm and the gated
+    // projection runs once, in its backward form, inside the MLP's backward (no gate | up in
+    // memory, no GLU backward kernel: 0.9 GB less traffic per 7B layer).
+    const bool defer = !keep && c->layer_type == 0;
+    if (defer) {
+      RC(lin_dx(s, dcur, m.d, bw.wdown, m.F, m.d, w.tmp.dact, m.F, nullptr, 0, m.T));
+      RC(hook_point(POINT_AFTER_DACT));
+    }
     if (!keep) {
       // full-block recompute of everything the backward reads
-      RC(block_forward(s, c, &bw, windows[l], cos_tables[l], sin_tables[l], xin, dnext, acts, false));
+      RC(block_forward(s, c, &bw, windows[l], cos_tables[l], sin_tables[l], xin, dnext, acts, false, true, defer));
     }
-    RC(block_backward(s, c, &bw, &bg, windows[l], cos_tables[l], sin_tables[l], xin, dcur, dnext, acts, w.tmp));
+    RC(block_backward(s, c, &bw, &bg, windows[l], cos_tables[l], sin_tables[l], xin, dcur, dnext, acts, w.tmp, defer));
     RC(ready(l));
     bf16* t = dcur;
     dcur = dnext;
@@ -924,6 +945,11 @@ extern "C" int32_t olmax_model_train_step(hipStream_t stream, hipStream_t opt_st
                step, lr, b1, b2, eps, wd, leaf_decay, hyper_dev, 0, {0, 0, 0, 0}, 0};
   x.head_windows = c->n_layers;  // one recompute window per layer
   x.layer_numel = per_layer_params(c);
+  // Pre-norm blocks open their backward with the d act GEMM (dY Wdown, hoisted in front of the
+  // recompute): its waves fill the register file, so an update running beside it would keep
+  // its workgroups off the CUs (measured: 1.9 ms instead of 0.5).  The update of the layer
+  // above therefore starts right behind that GEMM, beside the recompute's forward kernels.
+  if (c->layer_type == 0) x.flush_point = POINT_AFTER_DACT;
   // the optimizer stream must not run ahead of work already queued on the main stream
   int rc = OLMAX_OK;
   if (hipEventRecord(ev, stream) != hipSuccess || hipStreamWaitEvent(opt_stream, ev, 0) != hipSuccess)

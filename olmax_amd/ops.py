@@ -172,6 +172,23 @@ def gated_mlp_in(x, w_gate_up, act: str = "silu", gate_up_out=None, save_gate_up
     return out, gate_up_out
 
 
+def gated_mlp_in_bwd(x, w_gate_up, dact, act: str = "silu"):
+    """The gated projection re-run in a backward pass that kept nothing: from x, [Wgate; Wup] and
+    dact = d loss / d(act(gate) * up) returns (act_out [T, F], d gate | d up [T, 2F]); gate | up are
+    never written.  Equals gated_mlp_in followed by glu_bwd."""
+    _need_gpu(x, w_gate_up, dact)
+    x, dact = _rows2d(x), _rows2d(dact)
+    T, d = x.shape
+    F = w_gate_up.shape[0] // 2
+    assert dact.shape == (T, F) and dact.dtype == BF16
+    out = torch.empty(T, F, device=x.device, dtype=BF16)
+    dgu = torch.empty(T, 2 * F, device=x.device, dtype=BF16)
+    check(_L().olmax_gemm_glu_bwd_bf16(stream_ptr(), ptr(x), ptr(w_gate_up), ptr(dact), ptr(out), ptr(dgu), i32(T), i32(F),
+                                       i32(d), i64(x.stride(0)), i64(w_gate_up.stride(0)), i64(dact.stride(0)),
+                                       i64(out.stride(0)), i64(dgu.stride(0)), i32(_ACT[act])))
+    return out, dgu
+
+
 def qkv_rope_proj(x, w_qkv, cos, sin, *, rope_heads: int, seq_len: int, out=None):
     """q|k|v projection with RoPE applied to the first `rope_heads` heads (q then k, head_dim 128)
     in the GEMM epilogue (reference src/olmax/nn/attention.py:270-274, 298-300).  Returns [T, N]."""

@@ -257,6 +257,28 @@ def test_gated_mlp_in_fused_epilogue(act, T, F, d):
         assert maxrel(act_fused, want) < 2e-2
 
 
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("T,F,d", [(2048, 2048, 256), (4096, 1024, 128), (8192, 5504, 192), (96, 40, 24)])
+def test_gated_mlp_in_backward_form(act, T, F, d):
+    """The gated projection in its backward form (gate | up recomputed in the accumulators, the GLU
+    backward in the epilogue) must equal the forward-form GEMM followed by glu_bwd bit for bit: the
+    activation output and d gate | d up; odd shapes take the unfused path inside the call.  Against
+    the oracle on the shapes it can hold."""
+    ops = _ops()
+    say(f"gated_mlp_in backward form {act} T{T} F{F} d{d}")
+    x = bfr(T, d, seed=1); w = bfr(2 * F, d, seed=2, scale=d ** -0.5); dact = bfr(T, F, seed=3)
+    xc, wc, dc = x.cuda(), w.cuda(), dact.cuda()
+    act_plain, gu = ops.gated_mlp_in(xc, wc, act)
+    dg, du = ops.glu_bwd(gu[:, :F], gu[:, F:], dc, act)
+    act_b, dgu = ops.gated_mlp_in_bwd(xc, wc, dc, act)
+    assert torch.equal(act_b, act_plain)
+    assert torch.equal(dgu[:, :F], dg) and torch.equal(dgu[:, F:], du)
+    if T * F * d <= 2 ** 31:
+        gu_want = ref.linear_fwd(x.double(), w.double(), rt)
+        wg, wu = ref.glu_bwd(gu_want[:, :F], gu_want[:, F:], dact.double(), act)
+        check_close(dgu[:, :F], wg, "dgate", tol=3e-2); check_close(dgu[:, F:], wu, "dup", tol=3e-2)
+
+
 @pytest.mark.parametrize("T,S,H,KH,d", [(4096, 1024, 8, 8, 256), (8192, 4096, 6, 2, 192), (512, 256, 2, 2, 128), (8192, 2048, 5, 3, 128)])
 def test_qkv_projection_with_rope_in_the_epilogue(T, S, H, KH, d):
     """The q|k|v GEMM with RoPE in its epilogue must equal GEMM + qk_rope_fwd (in place on the q and
