@@ -26,6 +26,12 @@ extern "C" int32_t olmax_fill_zero(hipStream_t stream, void* p, int64_t nbytes);
 namespace {
 
 __device__ __forceinline__ float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// tanh(raw * scale / cap) from a raw score, with c1 = 2 * scale * log2(e) / cap formed once per
+// kernel: tanh(x) = 1 - 2 / (exp(2x) + 1) as one multiply, exp2, add, reciprocal and fma.  (Dividing
+// by cap per score, as the formula reads, costs a correctly rounded division per element.)
+__device__ __forceinline__ float cap_tanh(float raw, float c1) {
+  return __builtin_fmaf(-2.f, __builtin_amdgcn_rcpf(fexp2(raw * c1) + 1.f), 1.f);
+}
 
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
@@ -228,6 +234,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
     }
   };
   const float sc2 = scale * LOG2E;
+  const float cap_c1 = CAP ? 2.f * sc2 / cap : 0.f, cap_l2 = cap * LOG2E;  // soft-cap: see cap_tanh
   FragAddr fa;
   fa.init(lane);
 
@@ -258,7 +265,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(
 #pragma unroll
         for (int jt = 0; jt < 2; jt++)
 #pragma unroll
-          for (int r = 0; r < 16; r++) st[jt][r] = cap * fast_tanh(st[jt][r] * scale / cap) * LOG2E;
+          for (int r = 0; r < 16; r++) st[jt][r] = cap_l2 * cap_tanh(st[jt][r], cap_c1);
       }
       const bool need_mask = (j0 + 63 > iw0) || (window >= 0 && j0 < iw0 + 31 - window);
       if (need_mask) {
@@ -415,6 +422,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     }
   };
   const float sc2 = scale * LOG2E;
+  const float cap_c1 = CAP ? 2.f * sc2 / cap : 0.f, cap_l2 = cap * LOG2E;  // soft-cap: see cap_tanh
 
   FragAddr fa;
   fa.init(lane);
@@ -448,8 +456,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
         for (int r = 0; r < 16; r++) {
           float s = st[jt][r], chain = 1.f, p;
           if (CAP) {
-            const float th = fast_tanh(s * scale / cap);
-            p = fexp2(cap * th * LOG2E - lse2);
+            const float th = cap_tanh(s, cap_c1);
+            p = fexp2(__builtin_fmaf(th, cap_l2, -lse2));
             chain = 1.f - th * th;
           } else {
             p = fexp2(__builtin_fmaf(s, sc2, -lse2));
@@ -534,6 +542,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
   const int ntile = t_hi - t_lo + 1;
   const int total = ntile * rep;  // flattened (head, tile) iteration space
   const float sc2 = scale * LOG2E;
+  const float cap_c1 = CAP ? 2.f * sc2 / cap : 0.f, cap_l2 = cap * LOG2E;  // soft-cap: see cap_tanh
   const unsigned lds0 = lds_addr_of(smem);
   const int wv = __builtin_amdgcn_readfirstlane(wave);
 
@@ -616,8 +625,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(
           const int i = ib + il + e;
           float s = sa[r], chain = 1.f, p;
           if (CAP) {
-            const float th = fast_tanh(s * scale / cap);
-            p = fexp2(cap * th * LOG2E - l4[e]);
+            const float th = cap_tanh(s, cap_c1);
+            p = fexp2(__builtin_fmaf(th, cap_l2, -l4[e]));
             chain = 1.f - th * th;
           } else {
             p = fexp2(__builtin_fmaf(s, sc2, -l4[e]));

@@ -146,7 +146,7 @@ __device__ __forceinline__ float act_gelu(float g) {
 
 // derivatives of the two activations (the backward of act(gate) * up)
 __device__ __forceinline__ float act_silu_grad(float g) {
-  const float s = 1.f / (1.f + __expf(-g));
+  const float s = __builtin_amdgcn_rcpf(1.f + __expf(-g));  // as act_silu: hardware reciprocal, not a rounded division
   return s * (1.f + g * (1.f - s));
 }
 __device__ __forceinline__ float act_gelu_grad(float g) {

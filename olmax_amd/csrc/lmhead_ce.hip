@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
     float zl = 0.f;
     if (counted && inrange) {
       zl = Io<T>::ld1(zr + label);
-      if (CAP) zl = cap * tanhf(zl * inv_cap);
+      if (CAP) zl = cap * fast_tanh(zl * inv_cap);
     }
     label_logit = zl;
   }
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
     float cm = -INFINITY;
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
-      if (CAP) f[e] = cap * tanhf(f[e] * inv_cap);
+      if (CAP) f[e] = cap * fast_tanh(f[e] * inv_cap);
       cm = fmaxf(cm, f[e]);
     }
     if (cm > mx) {
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
   }
   for (int i = nvec * VEC + threadIdx.x; i < V; i += 256) {
     float f = Io<T>::ld1(zr + i);
-    if (CAP) f = cap * tanhf(f * inv_cap);
+    if (CAP) f = cap * fast_tanh(f * inv_cap);
     if (f > mx) {
       sm *= __expf(mx - f);
       mx = f;
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
     for (int e = 0; e < VEC; e++) {
       float z = f[e], chain = 1.f;
       if (CAP) {
-        const float t = tanhf(z * inv_cap);
+        const float t = fast_tanh(z * inv_cap);
         z = cap * t;
         chain = 1.f - t * t;
       }
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256) void ce_row_kernel(
   for (int i = nvec * VEC + threadIdx.x; i < V; i += 256) {
     float z = Io<T>::ld1(zr + i), chain = 1.f;
     if (CAP) {
-      const float t = tanhf(z * inv_cap);
+      const float t = fast_tanh(z * inv_cap);
       z = cap * t;
       chain = 1.f - t * t;
     }
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(THREADS) void ce_row_regs_kernel(
     float zl = 0.f;
     if (counted && inrange) {
       zl = bf2f(zr[label]);
-      if (CAP) zl = cap * tanhf(zl * inv_cap);
+      if (CAP) zl = cap * fast_tanh(zl * inv_cap);
     }
     label_logit = zl;
   }
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(THREADS) void ce_row_regs_kernel(
   }
   auto value = [&](bf16 x) {
     const float f = bf2f(x);
-    return CAP ? cap * tanhf(f * inv_cap) : f;
+    return CAP ? cap * fast_tanh(f * inv_cap) : f;
   };
   float mx = -INFINITY;
 #pragma unroll
@@ -234,7 +234,7 @@ __global__ __launch_bounds__(THREADS) void ce_row_regs_kernel(
       for (int e = 0; e < 8; e++) {
         float z = bf2f(c[i].e[e]), chain = 1.f;
         if (CAP) {
-          const float t = tanhf(z * inv_cap);
+          const float t = fast_tanh(z * inv_cap);
           z = cap * t;
           chain = 1.f - t * t;
         }

@@ -114,6 +114,38 @@ def test_gemm_256_tiles_row_strided_operands(M, N, K, al, bl):
     assert not out[:, :16].any() and not out[:, 16 + N:].any()  # nothing written outside the view
 
 
+@pytest.mark.parametrize("M,N,K,al,bl", [(8192, 3072, 256, 0, 0), (2048, 5120, 192, 0, 1), (4096, 2048, 320, 1, 1),
+                                          (2048 + 512, 2048 + 768, 128, 0, 0), (6144, 11008, 64, 1, 1)])
+def test_gemm_tile_order_does_not_change_results(M, N, K, al, bl):
+    """Which tile a workgroup takes is a scheduling choice (one run of tiles per XCD, or windows of
+    8 x 4 tiles dealt so that the XCDs cover 1, 2, 4 or 8 strips of tile rows together, on grids
+    that divide into windows and on grids that need padded windows and surplus workgroups): every
+    order must cover every tile exactly once, so the products are bit-identical."""
+    ops = _ops()
+    from olmax_amd import _lib
+    L = _lib.load()
+    say(f"gemm tile orders M{M} N{N} K{K} a{al} b{bl}")
+    a = bfr(*((M, K) if al == 0 else (K, M)), seed=21).cuda()
+    b = bfr(*((N, K) if bl == 0 else (K, N)), seed=22).cuda()
+    r = bfr(M, N, seed=23).cuda()
+    outs = []
+    try:
+        for order in (-1, 0, 1, 2, 4, 8):
+            L.olmax_gemm_set_order(order)
+            out = torch.full((M, N), float("nan"), device="cuda", dtype=BF)
+            ops.gemm(a, b, a_layout=al, b_layout=bl, residual=r, out=out)
+            outs.append(out)
+    finally:
+        L.olmax_gemm_set_order(0)
+    torch.cuda.synchronize()
+    assert not torch.isnan(outs[0].float()).any()
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+    af = a.double() if al == 0 else a.double().t()
+    bf_ = b.double() if bl == 0 else b.double().t()
+    assert maxrel(outs[0], (af @ bf_.t() + r.double()).cpu()) < 6e-3
+
+
 def test_gemm_rejects_bad_arguments():
     ops = _ops()
     from olmax_amd._lib import OlmaxHipError
