@@ -48,13 +48,17 @@ __device__ __forceinline__ int tile_off(int row, int c) { return row * 256 + ((c
 // Per-lane byte offsets of the operand fragments inside a [rows][128] tile.  The swizzle only
 // looks at row bits 0-3, so stepping rows by 16 or 32 is a plain immediate offset and the
 // eight (k-contiguous) plus eight (transposed) lane-dependent offsets are loop invariant.
-struct FragAddr {
-  int kc[8];     // row (lane % 32), k-step s
-  int tr[4][2];  // column tile dt, half h of the transposed read
+// LEAN: the k-contiguous offsets are formed at each read from the first one (kc[s] = kc[0] ^ 32 s:
+// the k-step only enters the XOR-swizzled chunk index) instead of living in eight registers, for a
+// kernel that would otherwise spill them.
+template <bool LEAN = false>
+struct FragAddrT {
+  int kc[LEAN ? 1 : 8];  // row (lane % 32), k-step s
+  int tr[4][2];          // column tile dt, half h of the transposed read
   __device__ __forceinline__ void init(int lane) {
     const int l32 = lane & 31, lhi = lane >> 5;
 #pragma unroll
-    for (int s = 0; s < 8; s++) kc[s] = l32 * 256 + (((2 * s + lhi) ^ swz(l32)) << 4);
+    for (int s = 0; s < (LEAN ? 1 : 8); s++) kc[s] = l32 * 256 + (((2 * s + lhi) ^ swz(l32)) << 4);
     const int j16 = lane & 15, g16 = lane >> 4;
 #pragma unroll
     for (int dt = 0; dt < 4; dt++)
@@ -67,7 +71,12 @@ struct FragAddr {
   }
   // k-contiguous fragment: rows row0 + lane%32 (row0 multiple of 16), k-step s
   __device__ __forceinline__ bf16x8 load_kc(const unsigned char* tile, int row0, int s) const {
-    return *reinterpret_cast<const bf16x8*>(tile + kc[s] + row0 * 256);
+    int off = kc[LEAN ? 0 : s];
+    if (LEAN) {
+      asm volatile("" : "+v"(off));  // keeps the XOR at the read: hoisted out of the loop it is a register again
+      off ^= s << 5;
+    }
+    return *reinterpret_cast<const bf16x8*>(tile + off + row0 * 256);
   }
   // transposed fragment: MFMA rows = storage columns dt*32 + lane%32, k = storage rows r0 + {..}
   __device__ __forceinline__ bf16x8 load_tr(const unsigned char* tile, int r0, int dt) const {
@@ -81,6 +90,7 @@ struct FragAddr {
     return p.v;
   }
 };
+typedef FragAddrT<false> FragAddr;
 
 // A/B operand fragment with the k index contiguous in storage: row `row`, k-step s (16 wide)
 __device__ __forceinline__ bf16x8 frag_kc(const unsigned char* tile, int row, int s, int lhi) {
@@ -141,24 +151,25 @@ __device__ __forceinline__ WgCoord decode_wg(int id, int ngroups, int rep) {
   return c;
 }
 
-// The same tile transfer with everything lane-dependent hoisted out of the loop: per-lane
-// byte offsets (row * ld + swizzled chunk) are computed once, a transfer is ROWS/16 DMA
-// instructions off a wave-uniform row pointer.  Only for tiles that lie entirely inside the
-// sequence (no row clamping).
+// The same tile transfer with everything lane-dependent hoisted out of the loop: a lane's byte
+// offset (row * ld + swizzled chunk) inside a 16-row group is computed once, and since the
+// swizzle only looks at row bits 0-3 the ROWS/16 DMA instructions of a transfer differ by a
+// wave-uniform 16 * ld elements, which goes into the scalar base: one vector register per
+// operand whatever the tile height.  Only for tiles that lie entirely inside the sequence (no
+// row clamping).
 template <int ROWS>
 struct TileDma {
-  unsigned off[ROWS / 16];
+  unsigned off;
+  int64_t step;
   __device__ __forceinline__ void init(int64_t ld, int wave, int lane) {
-#pragma unroll
-    for (int i = 0; i < ROWS / 16; i++) {
-      const int p = (i * 4 + wave) * 64 + lane;
-      const int row = p >> 4, ph = p & 15;
-      off[i] = (unsigned)((row * ld + ((ph ^ swz(row)) << 3)) * 2);
-    }
+    const int p = wave * 64 + lane;
+    const int row = p >> 4, ph = p & 15;
+    off = (unsigned)((row * ld + ((ph ^ swz(row)) << 3)) * 2);
+    step = 16 * ld;
   }
   __device__ __forceinline__ void issue(const bf16* row0, unsigned lds_addr, int wave) const {
 #pragma unroll
-    for (int i = 0; i < ROWS / 16; i++) dma16_s(row0, off[i], lds_addr + (i * 4 + wave) * 1024);
+    for (int i = 0; i < ROWS / 16; i++) dma16_s(row0 + i * step, off, lds_addr + (i * 4 + wave) * 1024);
   }
 };
 
@@ -424,7 +435,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
   const float sc2 = scale * LOG2E;
   const float cap_c1 = CAP ? 2.f * sc2 / cap : 0.f, cap_l2 = cap * LOG2E;  // soft-cap: see cap_tanh
 
-  FragAddr fa;
+  FragAddrT<CAP> fa;  // the soft-cap variant is the one short of registers
   fa.init(lane);
 
   load_kv(t_lo, 0);
@@ -439,22 +450,12 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
       const unsigned char* sk = smem + cur * 32768;
       const unsigned char* sv = sk + 16384;
       const bool need_mask = (j0 + 63 > iw0) || (window >= 0 && j0 < iw0 + 31 - window);
-      f32x16 st[2], dpt[2];
-#pragma unroll
-      for (int jt = 0; jt < 2; jt++) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) { st[jt][r] = 0.f; dpt[jt][r] = 0.f; }
-#pragma unroll
-        for (int s = 0; s < 8; s++) {
-          st[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(sk, jt * 32, s), qf[s], st[jt], 0, 0, 0);
-          dpt[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(sv, jt * 32, s), dof[s], dpt[jt], 0, 0, 0);
-        }
-      }
-#pragma unroll
-      for (int jt = 0; jt < 2; jt++)
+      // dS of one 32-key half from its scores and dP, packed as the B operand of the dQ product
+      bf16x8 dsb[4];
+      auto finish_half = [&](int jt, f32x16& sj, const f32x16& dpj) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          float s = st[jt][r], chain = 1.f, p;
+          float s = sj[r], chain = 1.f, p;
           if (CAP) {
             const float th = cap_tanh(s, cap_c1);
             p = fexp2(__builtin_fmaf(th, cap_l2, -lse2));
@@ -467,11 +468,29 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
             const bool ok = (j <= qi) && (window < 0 || j >= qi - window);
             p = ok ? p : 0.f;
           }
-          st[jt][r] = p * (dpt[jt][r] - dlt) * chain;
+          sj[r] = p * (dpj[r] - dlt) * chain;
         }
-      bf16x8 dsb[4];
+        dsb[2 * jt] = pack_bf16x8(sj, 0);
+        dsb[2 * jt + 1] = pack_bf16x8(sj, 8);
+      };
+      f32x16 st[2], dpt[2];
 #pragma unroll
-      for (int u = 0; u < 4; u++) dsb[u] = pack_bf16x8(st[u >> 1], (u & 1) * 8);
+      for (int jt = 0; jt < 2; jt++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) { st[jt][r] = 0.f; dpt[jt][r] = 0.f; }
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+          st[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(sk, jt * 32, s), qf[s], st[jt], 0, 0, 0);
+          dpt[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.load_kc(sv, jt * 32, s), dof[s], dpt[jt], 0, 0, 0);
+        }
+        // with the soft-cap's extra temporaries both halves do not fit the register file at once:
+        // finish each half before the next one's products start
+        if (CAP) finish_half(jt, st[jt], dpt[jt]);
+      }
+      if (!CAP) {
+#pragma unroll
+        for (int jt = 0; jt < 2; jt++) finish_half(jt, st[jt], dpt[jt]);
+      }
 #pragma unroll
       for (int u = 0; u < 4; u++)
 #pragma unroll
