@@ -50,6 +50,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(OlmaxAttnFwd, AttnFwd,
 static ffi::Error AttnBwd(hipStream_t st, Buf q, Buf k, Buf v, Buf o, Buf lse, Buf d_o, Out dq, Out dk, Out dv, Out ws,
                           int32_t window, float softcap) {
   auto d = q.dimensions();
+  if (d.size() != 4 || k.dimensions().size() != 4) return ffi::Error::InvalidArgument("olmax_attn_bwd: q/k/v must be [B,S,H,D]");
   const int32_t B = d[0], Sq = d[1], H = d[2], D = d[3], K = k.dimensions()[2];
   const int64_t hd = (int64_t)H * D, kd = (int64_t)K * D;
   return Status(olmax_attn_bwd(S(st), q.untyped_data(), k.untyped_data(), v.untyped_data(), o.untyped_data(),

@@ -196,7 +196,9 @@ def hip_lm_head_cross_entropy(h, weight, labels, final_softcap: float = 0.0):
 def _lm_head_vjp():
     jax, jnp = _jax()
 
-    @functools.partial(jax.custom_vjp, nondiff_argnums=(2, 3))
+    # labels is an array (a tracer under jit), so it is a regular argument with no cotangent, not a
+    # nondiff_argnums entry (those must be static Python values)
+    @functools.partial(jax.custom_vjp, nondiff_argnums=(3,))
     def head(h, w, labels, softcap):
         return fwd(h, w, labels, softcap)[0]
 
@@ -210,9 +212,9 @@ def _lm_head_vjp():
             h2, w, labels.reshape(-1).astype(jnp.int32), softcap=np.float32(softcap))
         return loss, (dh.reshape(h.shape), dw)
 
-    def bwd(labels, softcap, res, g):
+    def bwd(softcap, res, g):
         dh, dw = res
-        return (g * dh).astype(dh.dtype), (g * dw).astype(dw.dtype)
+        return (g * dh).astype(dh.dtype), (g * dw).astype(dw.dtype), None
 
     head.defvjp(fwd, bwd)
     return head
