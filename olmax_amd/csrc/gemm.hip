@@ -818,13 +818,14 @@ extern "C" int32_t olmax_gemm_profile_end_shapes(int32_t* keys, int32_t* mnk, do
 }
 
 static int device_cu_count() {
-  static int n = 0;
-  if (!n) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n = v;
-    else n = 256;
+  static std::atomic<int> n{0};  // every thread that finds 0 computes the same value
+  int v = n.load(std::memory_order_relaxed);
+  if (!v) {
+    int dev = 0;
+    if (!(hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)) v = 256;
+    n.store(v, std::memory_order_relaxed);
   }
-  return n;
+  return v;
 }
 
 extern "C" int32_t olmax_gemm_bf16(hipStream_t stream, const void* A, const void* B, void* C,
